@@ -423,6 +423,11 @@ typedef struct vra_model_config {
   int32_t sliding_window;
 } vra_model_config;
 
+/* vra_model_config.arch of a model that is a LIST OF LAYERS (vllm_rs_amd/host/stack_model.h): hidden_size = width, vocab_size, num_layers,
+ * dtype (VRA_BF16 or VRA_F32) and max_position_embeddings are read from the struct, everything else from the spec text of
+ * vra_engine_create_spec.  The Ditilix design loads as such a model. */
+#define VRA_ARCH_STACK 3
+
 typedef struct vra_engine_config {
   int32_t block_size;             /* 64 (config.rs:466) */
   int32_t max_num_seqs;           /* 0 = auto */
@@ -607,6 +612,21 @@ int32_t vra_engine_forward_tokens(void* eng, const uint32_t* h_ids, const int64_
                                   const uint32_t* h_context_lens, const uint32_t* h_cu_seqlens_q,
                                   int32_t n_seqs, int32_t stochastic, int32_t top_k, float top_p,
                                   float temperature, uint64_t seed, uint32_t* h_tokens_out);
+/* vra_engine_create for VRA_ARCH_STACK models: `spec` lists the layers (format: vllm_rs_amd/host/stack_model.h; written by
+ * vllm_rs_amd/checkpoint.py from a config.json).  Tensors then arrive through vra_engine_load_tensor under the checkpoint's names. */
+void* vra_engine_create_spec(const vra_model_config* mc, const vra_engine_config* ec, const char* spec);
+/* One step of a replayed trace: entry i brings h_counts[i] further tokens of request h_req[i] (concatenated in h_tokens) and asks for
+ * the logits at h_n_want[i] of them (indices into the entry, concatenated in h_want); all entries run as ONE batch.  A request is
+ * admitted at its first entry and keeps its pages in the engine's block manager until it appears in h_end (requests that end after
+ * this step).  h_logits_out: host [total wanted, vocab] f32 in entry / want order.  Returns the number of rows written, -1 on error. */
+int32_t vra_engine_replay_step(void* eng, int32_t n_entries, const int64_t* h_req, const int32_t* h_counts,
+                               const uint32_t* h_tokens, const int32_t* h_n_want, const int32_t* h_want,
+                               int32_t n_end, const int64_t* h_end, float* h_logits_out);
+/* parity instrumentation of layer-stack models: keep / read the residual stream after every layer run of the last forward,
+ * f32 [layer runs, tokens of the step, width]; read returns the bytes copied, -1 if the model class does not offer it */
+void vra_engine_debug_layer_trace(void* eng, int32_t on);
+int64_t vra_engine_debug_read_layer_trace(void* eng, void* h_out, int64_t max_bytes);
+
 /* decode-step microbenchmark hook used by bench.py: runs `steps` decode steps of the current
  * running batch back to back (graph replay when enabled) and returns elapsed ms measured with HIP
  * events on the engine stream; tokens are sampled and appended exactly as in vra_engine_step. */

@@ -197,6 +197,10 @@ def load():
     _sig(lib, "vra_pc_evict_blocks", c_i32, P, c_i32, P, c_i32)
     _sig(lib, "vra_engine_create", P, MC, EC)
     _sig(lib, "vra_engine_destroy", None, P)
+    _sig(lib, "vra_engine_create_spec", P, MC, EC, C.c_char_p)
+    _sig(lib, "vra_engine_replay_step", c_i32, P, c_i32, P, P, P, P, P, c_i32, P, P)
+    _sig(lib, "vra_engine_debug_layer_trace", None, P, c_i32)
+    _sig(lib, "vra_engine_debug_read_layer_trace", c_i64, P, P, c_i64)
     _sig(lib, "vra_engine_init_synthetic", c_i32, P)
     _sig(lib, "vra_engine_load_tensor", c_i32, P, C.c_char_p, P, P, c_i32, c_i32)
     _sig(lib, "vra_engine_finalize_weights", c_i32, P)

@@ -49,9 +49,63 @@ def read_safetensors(path):
     return out
 
 
+# Architectures whose config.json lists the layers one by one (key "architecture", a string): name -> parser to the dict of a
+# layer-stack model (vllm_rs_amd/host/stack_model.h).  Their tensors keep the checkpoint's own names.
+def _num(v):
+    return repr(float(v))
+
+
+def parse_ditilix(cfg_json, dtype=None):
+    """Ditilix config.json -> cfg dict with arch "stack": sizes for the engine plus the spec text (one `stack` record, one `layer`
+    record per entry of "layers") the native model class parses.  Every size and constant is taken from the config; keys the design
+    makes optional (q_temp, softcap, kv_from, mlp, shared) switch their mechanism off when absent or null."""
+    td = dtype or cfg_json.get("torch_dtype", "bfloat16")
+    dt = {"bfloat16": BF16, "bf16": BF16, "float32": F32, "f32": F32, BF16: BF16, F32: F32}.get(td)
+    if dt is None:
+        raise ValueError(f"dtype {td!r}: a layer stack runs in bfloat16 or float32")
+    norm = cfg_json.get("norm") or {}
+    width, vocab, layers = int(cfg_json["width"]), int(cfg_json["vocab"]), cfg_json["layers"]
+    lines = ["stack width=%d vocab=%d eps=%s groups=%d residual_mult=%s logit_scale=%s pos_base=%s" % (
+        width, vocab, _num(norm.get("eps", 1e-6)), int(norm.get("groups", 1)), _num(cfg_json.get("residual_mult", 1.0)),
+        _num(cfg_json.get("logit_scale", 1.0)), _num(10000.0))]
+    heads = kv_heads = dim = 1
+    for i, layer in enumerate(layers):
+        if layer.get("type", "attention") != "attention":
+            raise ValueError(f"layer {i}: mixer type {layer.get('type')!r} is not part of this design")
+        mx = layer["mixer"]
+        f = dict(heads=int(mx["heads"]), kv_heads=int(mx.get("kv_heads", mx["heads"])), dim=int(mx["dim"]), vdim=int(mx.get("vdim", mx["dim"])),
+                 scale=_num(mx["scale"]) if mx.get("scale") is not None else _num(int(mx["dim"]) ** -0.5),
+                 softcap=_num(mx.get("softcap") or 0.0), kv_from=int(mx["kv_from"]) if mx.get("kv_from") is not None else -1)
+        qt = mx.get("q_temp")
+        if qt:
+            f.update(temp_coef=_num(qt["coef"]), temp_every=int(qt["every"]))
+        mlp = layer.get("mlp")
+        if not mlp:
+            f.update(mlp="none")
+        elif mlp["kind"] == "dense":
+            f.update(mlp="dense", ff=int(mlp["ff"]))
+        elif mlp["kind"] == "moe":
+            f.update(mlp="moe", ff=int(mlp["expert"]["ff"]), limit=_num(mlp["expert"].get("limit") or 0.0),
+                     experts=int(mlp["router"]["experts"]), top=int(mlp["router"].get("top", 1)))
+            if mlp.get("shared"):
+                f.update(shared_ff=int(mlp["shared"]["ff"]), shared_limit=_num(mlp["shared"].get("limit") or 0.0))
+        else:
+            raise ValueError(f"layer {i}: feed-forward kind {mlp['kind']!r} is not part of this design")
+        lines.append("layer " + " ".join(f"{k}={v}" for k, v in f.items()))
+        heads, kv_heads, dim = max(heads, f["heads"]), max(kv_heads, f["kv_heads"]), max(dim, f["dim"], f["vdim"])
+    return dict(arch="stack", design="Ditilix", hidden_size=width, vocab_size=vocab, num_layers=len(layers), num_heads=heads, num_kv_heads=kv_heads,
+                head_dim=dim, intermediate_size=0, max_position_embeddings=int(cfg_json.get("max_position_embeddings", 1 << 20)),
+                rms_norm_eps=float(norm.get("eps", 1e-6)), rope_theta=10000.0, dtype=dt, quant_method=None, spec="\n".join(lines) + "\n")
+
+
+STACK_ARCHS = {"Ditilix": parse_ditilix}
+
+
 def parse_config(cfg_json, dtype=None):
     """HF config.json dict -> the dict `vllm_rs_amd.engine.model_config` consumes; raises on what the reference
-    rejects (src/utils/mod.rs:1303-1330)."""
+    rejects (src/utils/mod.rs:1303-1330).  A config that names one of STACK_ARCHS under "architecture" goes to that design's parser."""
+    if cfg_json.get("architecture") in STACK_ARCHS:
+        return STACK_ARCHS[cfg_json["architecture"]](cfg_json, dtype)
     archs = cfg_json.get("architectures") or ["LlamaForCausalLM"]
     if archs[0] not in ARCHS:
         raise ValueError(f"architecture {archs[0]} is not on this path (supported: {sorted(ARCHS)})")
@@ -106,6 +160,14 @@ def to_engine_tensor(name, a, kind, model_dtype):
     as 16-bit patterns of the MODEL dtype (scales/bias are f16 on disk even for bf16 models: wna16.rs:97-109)."""
     if kind in ("i32", "u32"):
         return np.ascontiguousarray(a).view(np.uint32)
+    if model_dtype == F32:  # 32-bit models (layer stacks): every float tensor widened exactly
+        if kind == "f32":
+            return np.ascontiguousarray(a, np.float32)
+        if kind == "bf16":
+            return np.ascontiguousarray((a.astype(np.uint32) << 16).view(np.float32))
+        if kind == "f16":
+            return a.view(np.float16).astype(np.float32)
+        raise ValueError(f"{name}: cannot convert {kind} to float32")
     want = "bf16" if model_dtype == BF16 else "f16"
     if kind == want:
         return np.ascontiguousarray(a)

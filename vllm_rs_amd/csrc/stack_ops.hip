@@ -1,0 +1,703 @@
+// stack_ops.hip — operators of config-driven layer stacks (host/stack_model.cpp; every operator is specified in stack_launch.h), gfx950.
+//
+// What is kept in f32 whatever the storage type: positions and angles, norms, router logits and weights, attention scores and
+// softmax weights (the value product included: p stays f32, v is widened), the residual stream and every sum into it.
+// Matrix products: bf16 operands on v_mfma_f32_16x16x32_bf16 with f32 accumulation, or f32 operands on FMA (VRA_F32: no reduced
+// matrix mode anywhere).  Every reduction has an order that depends on the shapes of the model alone — never on the number of rows
+// of a step, on a row's place in the batch or on the pages it uses — so a token's result does not depend on how its prompt was cut.
+#include <math.h>
+
+#include "common.cuh"
+#include "stack_launch.h"
+
+namespace {
+
+template <typename T>
+struct El;
+template <>
+struct El<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float rnd(float v) { return v; }
+};
+template <>
+struct El<uint16_t> {
+  static __device__ __forceinline__ float ld(const uint16_t* p) { return BF16::to_f32(*p); }
+  static __device__ __forceinline__ void st(uint16_t* p, float v) { *p = BF16::from_f32(v); }
+  static __device__ __forceinline__ float rnd(float v) { return BF16::to_f32(BF16::from_f32(v)); }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float gated_pair(float g, float u, float limit, float act_alpha) {
+  if (limit > 0.f) {
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+  }
+  return g * sigmoidf_(act_alpha * g) * (u + 1.f);
+}
+
+// ------------------------------------------------------------------------------------------------ embedding + positions
+template <typename T>
+__global__ __launch_bounds__(256) void stk_embed_sinpos_kernel(const uint32_t* ids, const int64_t* pos, const T* embed, const float* inv_freq, float* x,
+                                                               int W, int V) {
+  const int t = blockIdx.x;
+  uint32_t id = ids[t];
+  if (id >= (uint32_t)V) id = 0;
+  const float p = (float)pos[t];
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float ang = p * inv_freq[c >> 1];
+    const float pe = (c & 1) ? cosf(ang) : sinf(ang);
+    x[(size_t)t * W + c] = El<T>::ld(embed + (size_t)id * W + c) + pe;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ grouped RMS norm (+ router)
+template <typename T>
+__global__ __launch_bounds__(256) void stk_group_norm_kernel(StkNormArgs a) {
+  extern __shared__ float lds[];
+  float* xs = lds;                      // [W] the row, then the normalised row
+  float* rs = lds + a.W;                // [groups] 1 / rms
+  float* zs = rs + a.groups;            // [n_router + gate_row]
+  const int t = blockIdx.x, W = a.W, gs = W / a.groups;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const float* x = a.x + (size_t)t * W;
+  for (int c = threadIdx.x; c < W; c += 256) xs[c] = x[c];
+  __syncthreads();
+  for (int g = wave; g < a.groups; g += 4) {
+    float s = 0.f;
+    for (int c = lane; c < gs; c += 64) {
+      const float v = xs[g * gs + c];
+      s = fmaf(v, v, s);
+    }
+    s = wave_sum(s);
+    if (lane == 0) rs[g] = 1.f / sqrtf(s / (float)gs + a.eps);
+  }
+  __syncthreads();
+  T* h = (T*)a.h + (size_t)t * W;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    const float v = xs[c] * rs[c / gs] * a.w[c];
+    xs[c] = v;
+    El<T>::st(h + c, v);
+  }
+  if (!a.router_w) return;
+  __syncthreads();
+  const int nz = a.n_router + (a.gate_row ? 1 : 0);
+  const T* rw = (const T*)a.router_w;
+  for (int e = wave; e < nz; e += 4) {
+    float s = 0.f;
+    for (int c = lane; c < W; c += 64) s = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), s);
+    s = wave_sum(s);
+    if (lane == 0) zs[e] = s;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    for (int j = 0; j < a.top; j++) {
+      int best = -1;
+      float bz = -INFINITY;
+      for (int e = 0; e < a.n_router; e++) {
+        bool taken = false;
+        for (int q = 0; q < j; q++) taken = taken || a.pair_expert[(size_t)t * a.top + q] == e;
+        if (!taken && (best < 0 || zs[e] > bz)) best = e, bz = zs[e];
+      }
+      a.pair_expert[(size_t)t * a.top + j] = best;
+      a.pair_weight[(size_t)t * a.top + j] = sigmoidf_(bz);
+    }
+    if (a.gate_row) a.gate_out[t] = sigmoidf_(zs[a.n_router]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ MoE rows sorted by expert
+__global__ __launch_bounds__(1024) void stk_moe_sort_kernel(const int* pair_expert, const float* pair_weight, int P, int top, int n_groups, int granule,
+                                                            int max_rows, int* row_token, float* row_scale, int* row_pair, int* tile_group) {
+  extern __shared__ int sl[];
+  int* counts = sl;
+  int* offs = sl + n_groups;
+  int* cursor = offs + n_groups;
+  const int tid = threadIdx.x;
+  for (int e = tid; e < n_groups; e += 1024) counts[e] = 0, cursor[e] = 0;
+  for (int r = tid; r < max_rows; r += 1024) row_token[r] = -1, row_pair[r] = -1, row_scale[r] = 0.f;
+  for (int t = tid; t < max_rows / granule; t += 1024) tile_group[t] = -1;
+  __syncthreads();
+  for (int p = tid; p < P; p += 1024) {
+    const int e = pair_expert[p];
+    if (e >= 0 && e < n_groups) atomicAdd(&counts[e], 1);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int off = 0;
+    for (int e = 0; e < n_groups; e++) {
+      offs[e] = off;
+      const int nt = (counts[e] + granule - 1) / granule;
+      for (int t = 0; t < nt; t++) tile_group[off / granule + t] = e;
+      off += nt * granule;
+    }
+  }
+  __syncthreads();
+  for (int p = tid; p < P; p += 1024) {
+    const int e = pair_expert[p];
+    if (e < 0 || e >= n_groups) continue;
+    const int r = offs[e] + atomicAdd(&cursor[e], 1);
+    row_token[r] = p / top;
+    row_scale[r] = pair_weight[p];
+    row_pair[r] = p;
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ GEMM, f32 FMA (any shape)
+// 256 threads: 16 (m) x 16 (n) threads, RM rows x 4 columns each; K in steps of 16 through LDS; k ascending: one fixed order.
+template <typename T, int RM>
+__global__ __launch_bounds__(256) void stk_gemm_simple_kernel(StkGemmArgs g) {
+  constexpr int TM = 16 * RM;
+  __shared__ float As[16][TM + 1];
+  __shared__ float Ws[16][65];
+  __shared__ int a_idx[TM];
+  __shared__ float a_sc[TM];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.x * TM, n0 = blockIdx.y * 64;
+  int group = 0;
+  if (g.tile_group) {
+    group = g.tile_group[blockIdx.x];
+    if (group < 0) return;
+  }
+  const T* A = (const T*)g.a;
+  const T* Wt = (const T*)g.w + (int64_t)group * g.w_group_stride;
+  if (tid < TM) {
+    const int r = m0 + tid;
+    int idx = r < g.M ? (g.a_row ? g.a_row[r] : r) : -1;
+    a_idx[tid] = idx;
+    a_sc[tid] = g.a_scale && idx >= 0 ? g.a_scale[r] : 1.f;
+  }
+  __syncthreads();
+  float acc[RM][4];
+  for (int i = 0; i < RM; i++)
+    for (int j = 0; j < 4; j++) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < g.K; k0 += 16) {
+    for (int i = tid; i < TM * 16; i += 256) {
+      const int r = i >> 4, kk = i & 15, idx = a_idx[r];
+      float v = 0.f;
+      if (idx >= 0 && k0 + kk < g.K) {
+        v = El<T>::ld(A + (int64_t)idx * g.lda + k0 + kk);
+        if (g.a_scale) v = El<T>::rnd(v * a_sc[r]);
+      }
+      As[kk][r] = v;
+    }
+    for (int i = tid; i < 64 * 16; i += 256) {
+      const int n = i >> 4, kk = i & 15;
+      Ws[kk][n] = (n0 + n < g.N && k0 + kk < g.K) ? El<T>::ld(Wt + (int64_t)(n0 + n) * g.K + k0 + kk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < 16; kk++) {
+      float av[RM], wv[4];
+      for (int i = 0; i < RM; i++) av[i] = As[kk][ty * RM + i];
+      for (int j = 0; j < 4; j++) wv[j] = Ws[kk][tx * 4 + j];
+      for (int i = 0; i < RM; i++)
+        for (int j = 0; j < 4; j++) acc[i][j] = fmaf(av[i], wv[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+  for (int i = 0; i < RM; i++) {
+    const int r = m0 + ty * RM + i;
+    if (r >= g.M || a_idx[ty * RM + i] < 0) continue;
+    const int orow = g.out_row ? g.out_row[r] : r;
+    if (orow < 0) continue;
+    for (int j = 0; j < 4; j++) {
+      const int n = n0 + tx * 4 + j;
+      if (n >= g.N) continue;
+      const float v = acc[i][j] * g.alpha;
+      if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = v;
+      else El<T>::st((T*)g.out + (int64_t)orow * g.ldo + n, v);
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ GEMM, bf16 MFMA (K % 8 == 0)
+// A wave owns MT x NT tiles of 16 x 16; both operands come straight from global memory in the instruction's operand order (lane =
+// (row rq = lane & 15, k octet oct = lane >> 4): 16 bytes of one row per lane and K-step of 32), the weights as the A operand and the
+// activations as B, so a lane ends up with 4 consecutive output columns of ONE activation row.  K ascending in steps of 32.
+template <int MT, int NT, int WM, int WN, bool SCALED>
+__global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs g) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int wm = wave % WM, wn = wave / WM, rq = lane & 15, oct = lane >> 4;
+  int group = 0;
+  if (g.tile_group) {
+    group = g.tile_group[blockIdx.x];
+    if (group < 0) return;
+  }
+  const uint16_t* A = (const uint16_t*)g.a;
+  const uint16_t* Wt = (const uint16_t*)g.w + (int64_t)group * g.w_group_stride;
+  const int m_base = blockIdx.x * (16 * MT * WM) + wm * 16 * MT;
+  const int n_base = blockIdx.y * (16 * NT * WN) + wn * 16 * NT;
+  const uint16_t* ap[MT];
+  const uint16_t* wp[NT];
+  bool av[MT], wv[NT];
+  float asc[MT];
+  for (int mt = 0; mt < MT; mt++) {
+    const int r = m_base + mt * 16 + rq;
+    const int idx = r < g.M ? (g.a_row ? g.a_row[r] : r) : -1;
+    av[mt] = idx >= 0;
+    ap[mt] = A + (int64_t)(idx >= 0 ? idx : 0) * g.lda;
+    asc[mt] = SCALED && idx >= 0 ? g.a_scale[r] : 1.f;
+  }
+  for (int nt = 0; nt < NT; nt++) {
+    const int n = n_base + nt * 16 + rq;
+    wv[nt] = n < g.N;
+    wp[nt] = Wt + (int64_t)(n < g.N ? n : 0) * g.K;
+  }
+  f32x4 acc[MT][NT];
+  for (int mt = 0; mt < MT; mt++)
+    for (int nt = 0; nt < NT; nt++) acc[mt][nt] = vra_zero_acc();
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  for (int k0 = 0; k0 < g.K; k0 += 32) {
+    const int k = k0 + oct * 8;
+    const bool kin = k < g.K;
+    const int kc = kin ? k : 0;
+    u32x4 af[MT], wf[NT];
+    for (int mt = 0; mt < MT; mt++) {
+      u32x4 v = *(const u32x4*)(ap[mt] + kc);
+      if (SCALED) {
+        const float s = asc[mt];
+        for (int i = 0; i < 4; i++) {
+          const float lo = __uint_as_float(v[i] << 16) * s, hi = __uint_as_float(v[i] & 0xffff0000u) * s;
+          v[i] = BF16::pack2(lo, hi);
+        }
+      }
+      af[mt] = (av[mt] && kin) ? v : zero4;
+    }
+    for (int nt = 0; nt < NT; nt++) {
+      const u32x4 v = *(const u32x4*)(wp[nt] + kc);
+      wf[nt] = (wv[nt] && kin) ? v : zero4;
+    }
+    for (int mt = 0; mt < MT; mt++)
+      for (int nt = 0; nt < NT; nt++) BF16::mfma(acc[mt][nt], __builtin_bit_cast(s16x8, wf[nt]), __builtin_bit_cast(s16x8, af[mt]));
+  }
+  VRA_MFMA_DRAIN();
+  // lane: activation row rq of tile mt, output columns oct * 4 + j of tile nt
+  for (int mt = 0; mt < MT; mt++) {
+    const int r = m_base + mt * 16 + rq;
+    if (r >= g.M || !av[mt]) continue;
+    const int orow = g.out_row ? g.out_row[r] : r;
+    if (orow < 0) continue;
+    if (g.epi == 1) {
+      for (int nt = 0; nt + 1 < NT; nt += 2)
+        for (int j = 0; j < 4; j++) {
+          const int n = (n_base + nt * 16) / 2 + oct * 4 + j;
+          if (n >= g.N / 2) continue;
+          const float y = gated_pair(acc[mt][nt][j], acc[mt][nt + 1][j], g.limit, g.act_alpha);
+          if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = y;
+          else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(y);
+        }
+    } else {
+      for (int nt = 0; nt < NT; nt++)
+        for (int j = 0; j < 4; j++) {
+          const int n = n_base + nt * 16 + oct * 4 + j;
+          if (n >= g.N) continue;
+          const float v = acc[mt][nt][j] * g.alpha;
+          if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = v;
+          else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(v);
+        }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ activations
+template <typename T>
+__global__ __launch_bounds__(256) void stk_gated_act_kernel(const float* gu, T* out, int F, float limit, float act_alpha) {
+  const int m = blockIdx.x;
+  const int Fp = (F + 15) / 16 * 16;
+  for (int f = threadIdx.x; f < F; f += 256) {
+    const int b = f >> 4, i = f & 15;
+    const float gv = gu[(size_t)m * 2 * Fp + (2 * b) * 16 + i], uv = gu[(size_t)m * 2 * Fp + (2 * b + 1) * 16 + i];
+    El<T>::st(out + (size_t)m * Fp + f, gated_pair(gv, uv, limit, act_alpha));
+  }
+  for (int f = F + threadIdx.x; f < Fp; f += 256) El<T>::st(out + (size_t)m * Fp + f, 0.f);
+}
+
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+template <typename T>
+__global__ __launch_bounds__(256) void stk_polynorm_kernel(const float* z, T* out, const float* coef, int F, float eps) {
+  __shared__ float red[4];
+  const int m = blockIdx.x;
+  const float* zr = z + (size_t)m * F;
+  float s1 = 0.f, s2 = 0.f, s3 = 0.f;
+  for (int f = threadIdx.x; f < F; f += 256) {
+    const float v = zr[f], v2 = v * v, v3 = v2 * v;
+    s1 = fmaf(v, v, s1), s2 = fmaf(v2, v2, s2), s3 = fmaf(v3, v3, s3);
+  }
+  s1 = block_sum256(s1, red);
+  s2 = block_sum256(s2, red);
+  s3 = block_sum256(s3, red);
+  const float r1 = 1.f / sqrtf(s1 / (float)F + eps), r2 = 1.f / sqrtf(s2 / (float)F + eps), r3 = 1.f / sqrtf(s3 / (float)F + eps);
+  const float ca = coef[0], cb = coef[1], cc = coef[2], ce = coef[3];
+  for (int f = threadIdx.x; f < F; f += 256) {
+    const float v = zr[f], v2 = v * v, v3 = v2 * v;
+    El<T>::st(out + (size_t)m * F + f, ca * (v * r1) + cb * (v2 * r2) + cc * (v3 * r3) + ce);
+  }
+}
+
+__global__ __launch_bounds__(256) void stk_residual_combine_kernel(float* x, const float* o, const float* p1, int n1, const float* p2, const float* gate,
+                                                                   float mult, int W) {
+  const int t = blockIdx.x;
+  const float gt = gate ? gate[t] : 1.f;
+  for (int c = threadIdx.x; c < W; c += 256) {
+    float s = o ? o[(size_t)t * W + c] : 0.f;
+    for (int j = 0; j < n1; j++) s += p1[((size_t)t * n1 + j) * W + c];
+    if (p2) s += gt * p2[(size_t)t * W + c];
+    x[(size_t)t * W + c] += mult * s;
+  }
+}
+
+__global__ __launch_bounds__(256) void stk_gather_rows_kernel(const float* src, const uint32_t* rows, float* dst, int W) {
+  const int r = blockIdx.x;
+  const float* s = src + (size_t)rows[r] * W;
+  for (int c = threadIdx.x; c < W; c += 256) dst[(size_t)r * W + c] = s[c];
+}
+
+// ------------------------------------------------------------------------------------------------ paged KV cache
+template <typename T>
+__global__ __launch_bounds__(256) void stk_kv_store_kernel(const T* k, const T* v, int ld, T* kc, T* vc, const int64_t* slots, int kdim, int vdim) {
+  const int t = blockIdx.x;
+  const int64_t s = slots[t];
+  if (s < 0) return;
+  for (int c = threadIdx.x; c < kdim; c += 256) kc[s * kdim + c] = k[(size_t)t * ld + c];
+  for (int c = threadIdx.x; c < vdim; c += 256) vc[s * vdim + c] = v[(size_t)t * ld + c];
+}
+
+__device__ __forceinline__ float q_temperature(int64_t p, float coef, int every) {
+  if (every <= 0 || coef == 0.f) return 1.f;
+  return 1.f + coef * logf((float)((p + 1) / every) + 1.f);
+}
+__device__ __forceinline__ float cap_score(float s, float softcap) { return softcap > 0.f ? softcap * tanhf(s / softcap) : s; }
+
+// Portions of prompts (and whatever else shares their step): 16 query rows of one head per workgroup, 4 per wave; key tiles of KT
+// tokens staged once in LDS (f32) for all 16 rows; lane = key for the scores, lane = value channel for the weighted sum.
+// Tiles start at key 0 of the sequence and a row's running maximum / sum go tile by tile: the order does not depend on the portion.
+#define STK_QT 16
+template <typename T, int KT>
+__global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
+  extern __shared__ float lds[];
+  const int dim = a.dim, vdim = a.vdim, kld = dim + 1;
+  float* qs = lds;                      // [16][dim]  q * temp
+  float* ks = qs + STK_QT * dim;        // [KT][dim + 1]
+  float* vs = ks + KT * kld;            // [KT][vdim]
+  float* ps = vs + KT * vdim;           // [16][KT]
+  const int b = blockIdx.y, h = blockIdx.z, g = h / (a.H / a.G);
+  const int q0 = a.cu_q[b], q1 = a.cu_q[b + 1];
+  const int t0 = q0 + blockIdx.x * STK_QT;
+  if (t0 >= q1) return;
+  const int nq = min(STK_QT, q1 - t0);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const T* q = (const T*)a.q;
+  for (int i = tid; i < STK_QT * dim; i += 256) {
+    const int r = i / dim, d = i % dim;
+    float v = 0.f;
+    if (r < nq) v = El<T>::ld(q + (size_t)(t0 + r) * a.ldq + h * dim + d) * q_temperature(a.positions[t0 + r], a.temp_coef, a.temp_every);
+    qs[i] = v;
+  }
+  int64_t pq[4];
+  int64_t pmax = -1;
+  for (int i = 0; i < 4; i++) {
+    const int r = wave * 4 + i;
+    pq[i] = r < nq ? a.positions[t0 + r] : -1;
+  }
+  for (int r = 0; r < nq; r++) pmax = max(pmax, a.positions[t0 + r]);
+  const int n_keys = (int)min((int64_t)a.context_lens[b], pmax + 1);
+  float m[4], l[4], acc[4][4];
+  for (int i = 0; i < 4; i++) {
+    m[i] = -INFINITY, l[i] = 0.f;
+    for (int r = 0; r < 4; r++) acc[i][r] = 0.f;
+  }
+  const T* kc = (const T*)a.kc;
+  const T* vc = (const T*)a.vc;
+  const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
+  const int kdim = a.G * dim, vd_all = a.G * vdim;
+  for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
+    __syncthreads();
+    for (int i = tid; i < KT * dim; i += 256) {
+      const int j = i / dim, d = i % dim, key = kt0 + j;
+      float v = 0.f;
+      if (key < n_keys) {
+        const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
+        v = El<T>::ld(kc + slot * kdim + g * dim + d);
+      }
+      ks[j * kld + d] = v;
+    }
+    for (int i = tid; i < KT * vdim; i += 256) {
+      const int j = i / vdim, d = i % vdim, key = kt0 + j;
+      float v = 0.f;
+      if (key < n_keys) {
+        const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
+        v = El<T>::ld(vc + slot * vd_all + g * vdim + d);
+      }
+      vs[i] = v;
+    }
+    __syncthreads();
+    for (int i = 0; i < 4; i++) {
+      const int r = wave * 4 + i;
+      float s = -INFINITY;
+      if (lane < KT && pq[i] >= 0 && kt0 + lane <= pq[i] && kt0 + lane < n_keys) {
+        float d0 = 0.f;
+        for (int d = 0; d < dim; d++) d0 = fmaf(qs[r * dim + d], ks[lane * kld + d], d0);
+        s = cap_score(d0 * a.scale, a.softcap);
+      }
+      const float mn = fmaxf(m[i], wave_max(s));
+      float p = 0.f, corr = 1.f;
+      if (mn > -INFINITY) {
+        p = s > -INFINITY ? expf(s - mn) : 0.f;
+        corr = m[i] > -INFINITY ? expf(m[i] - mn) : 0.f;
+      }
+      l[i] = l[i] * corr + wave_sum(p);
+      m[i] = mn;
+      for (int rr = 0; rr < 4; rr++) acc[i][rr] *= corr;
+      if (lane < KT) ps[r * KT + lane] = p;
+    }
+    __syncthreads();
+    for (int rr = 0; rr < 4; rr++) {
+      const int d = lane + 64 * rr;
+      if (d >= vdim) break;
+      for (int j = 0; j < KT; j++) {
+        const float v = vs[j * vdim + d];
+        for (int i = 0; i < 4; i++) acc[i][rr] = fmaf(ps[(wave * 4 + i) * KT + j], v, acc[i][rr]);
+      }
+    }
+  }
+  T* out = (T*)a.out;
+  for (int i = 0; i < 4; i++) {
+    const int r = wave * 4 + i;
+    if (r >= nq) continue;
+    const float inv = l[i] > 0.f ? 1.f / l[i] : 0.f;
+    for (int rr = 0; rr < 4; rr++) {
+      const int d = lane + 64 * rr;
+      if (d < vdim) El<T>::st(out + (size_t)(t0 + r) * a.H * vdim + h * vdim + d, acc[i][rr] * inv);
+    }
+  }
+}
+
+// One decoded token per sequence: a workgroup per (sequence, query head); its 4 waves take the 64-key tiles of the context in turn,
+// read K rows straight from the cache (lane = key) and V rows channel-wise (lane = channel), and meet once in LDS.
+template <typename T>
+__global__ __launch_bounds__(256) void stk_attn_decode_kernel(StkAttnArgs a) {
+  extern __shared__ float lds[];
+  const int dim = a.dim, vdim = a.vdim;
+  float* qs = lds;                 // [dim]
+  float* ps = qs + dim;            // [4][64]
+  float* ms = ps + 4 * 64;         // [4] max, [4] sum
+  float* os = ms + 8;              // [4][vdim]
+  const int b = blockIdx.x, h = blockIdx.y, g = h / (a.H / a.G);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t p = a.positions[b];
+  const int n_keys = (int)min((int64_t)a.context_lens[b], p + 1);
+  const T* q = (const T*)a.q + (size_t)b * a.ldq + h * dim;
+  const float temp = q_temperature(p, a.temp_coef, a.temp_every);
+  for (int d = tid; d < dim; d += 256) qs[d] = El<T>::ld(q + d) * temp;
+  __syncthreads();
+  const T* kc = (const T*)a.kc;
+  const T* vc = (const T*)a.vc;
+  const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
+  const int kdim = a.G * dim, vd_all = a.G * vdim;
+  float m = -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int kt0 = wave * 64; kt0 < n_keys; kt0 += 4 * 64) {
+    const int key = kt0 + lane;
+    float s = -INFINITY;
+    if (key < n_keys) {
+      const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
+      const T* kr = kc + slot * kdim + g * dim;
+      float d0 = 0.f;
+      for (int d = 0; d < dim; d++) d0 = fmaf(qs[d], El<T>::ld(kr + d), d0);
+      s = cap_score(d0 * a.scale, a.softcap);
+    }
+    const float mn = fmaxf(m, wave_max(s));  // (the tile's first key exists: mn is finite)
+    const float pj = s > -INFINITY ? expf(s - mn) : 0.f;
+    const float corr = m > -INFINITY ? expf(m - mn) : 0.f;
+    l = l * corr + wave_sum(pj);
+    m = mn;
+    ps[wave * 64 + lane] = pj;
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int nj = min(64, n_keys - kt0);
+    for (int rr = 0; rr < 4; rr++) {
+      const int d = lane + 64 * rr;
+      if (d >= vdim) break;
+      float o = acc[rr] * corr;
+      for (int j = 0; j < nj; j++) {
+        const int kj = kt0 + j;
+        const int64_t slot = (int64_t)bt[kj / a.BS] * a.BS + kj % a.BS;
+        o = fmaf(ps[wave * 64 + j], El<T>::ld(vc + slot * vd_all + g * vdim + d), o);
+      }
+      acc[rr] = o;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  }
+  if (lane == 0) ms[wave] = m, ms[4 + wave] = l;
+  for (int rr = 0; rr < 4; rr++) {
+    const int d = lane + 64 * rr;
+    if (d < vdim) os[wave * vdim + d] = acc[rr];
+  }
+  __syncthreads();
+  const float M = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
+  T* out = (T*)a.out + (size_t)b * a.H * vdim + h * vdim;
+  for (int d = tid; d < vdim; d += 256) {
+    float L = 0.f, o = 0.f;
+    for (int w = 0; w < 4; w++) {
+      const float c = ms[w] > -INFINITY ? expf(ms[w] - M) : 0.f;
+      L += ms[4 + w] * c;
+      o += os[w * vdim + d] * c;
+    }
+    El<T>::st(out + d, L > 0.f ? o / L : 0.f);
+  }
+}
+
+template <typename F>
+void launch_checked(const char* what, F f) {
+  f();
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) vra_set_error("%s: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace
+
+// ================================================================================================ launchers
+int vra_stack_gemm_granule(int rows, int groups) { return groups > 0 && rows / groups >= 128 ? 64 : 16; }
+
+void vra_stack_gemm(const StkGemmArgs& g, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(g.a && g.w && g.out && g.M > 0 && g.N > 0 && g.K > 0, "stack gemm: null pointer or empty shape");
+  VRA_CHECK_ARG(dtype == VRA_BF16 || dtype == VRA_F32, "stack gemm: dtype must be bf16 or f32");
+  VRA_CHECK_ARG(!g.tile_group || g.granule == 16 || g.granule == 64, "stack gemm: granule must be 16 or 64");
+  hipStream_t st = as_stream(stream);
+  const bool big = g.tile_group ? g.granule == 64 : g.M > 32;
+  const bool mfma = dtype == VRA_BF16 && g.K % 8 == 0 && g.lda % 8 == 0 && ((uintptr_t)g.a % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
+                    (g.w_group_stride % 8 == 0);
+  VRA_CHECK_ARG(g.epi == 0 || (mfma && g.N % 32 == 0), "stack gemm: the gated epilogue needs the bf16 MFMA path and whole gate / up blocks");
+  if (mfma) {
+    if (big) {
+      dim3 grid((g.M + 63) / 64, (g.N + 127) / 128);
+      if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, true><<<grid, 256, 0, st>>>(g); });
+      else launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, false><<<grid, 256, 0, st>>>(g); });
+    } else {
+      dim3 grid((g.M + 15) / 16, (g.N + 63) / 64);
+      if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<1, 2, 1, 2, true><<<grid, 128, 0, st>>>(g); });
+      else launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<1, 2, 1, 2, false><<<grid, 128, 0, st>>>(g); });
+    }
+    return;
+  }
+  if (big) {
+    dim3 grid((g.M + 63) / 64, (g.N + 63) / 64);
+    if (dtype == VRA_F32) launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<float, 4><<<grid, 256, 0, st>>>(g); });
+    else launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<uint16_t, 4><<<grid, 256, 0, st>>>(g); });
+  } else {
+    dim3 grid((g.M + 15) / 16, (g.N + 63) / 64);
+    if (dtype == VRA_F32) launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<float, 1><<<grid, 256, 0, st>>>(g); });
+    else launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<uint16_t, 1><<<grid, 256, 0, st>>>(g); });
+  }
+}
+
+void vra_stack_embed_sinpos(const uint32_t* ids, const int64_t* positions, const void* embed, const float* inv_freq, float* x, int T, int W, int V,
+                            int dtype, int64_t stream) {
+  VRA_CHECK_ARG(ids && positions && embed && inv_freq && x && T > 0 && W > 0, "stack embed: null pointer or empty shape");
+  if (dtype == VRA_F32)
+    launch_checked("stack embed", [&] { stk_embed_sinpos_kernel<float><<<T, 256, 0, as_stream(stream)>>>(ids, positions, (const float*)embed, inv_freq, x, W, V); });
+  else
+    launch_checked("stack embed", [&] { stk_embed_sinpos_kernel<uint16_t><<<T, 256, 0, as_stream(stream)>>>(ids, positions, (const uint16_t*)embed, inv_freq, x, W, V); });
+}
+
+void vra_stack_group_norm(const StkNormArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.x && a.w && a.h && a.T > 0 && a.W > 0, "stack norm: null pointer or empty shape");
+  VRA_CHECK_ARG(a.groups >= 1 && a.W % a.groups == 0, "stack norm: the width must split into equal groups");
+  VRA_CHECK_ARG(!a.router_w || (a.pair_expert && a.pair_weight && a.top >= 1 && a.top <= a.n_router && (!a.gate_row || a.gate_out)), "stack norm: router outputs");
+  const size_t lds = ((size_t)a.W + a.groups + a.n_router + 2) * sizeof(float);
+  VRA_CHECK_ARG(lds <= 64 * 1024, "stack norm: row does not fit LDS");
+  if (dtype == VRA_F32) launch_checked("stack norm", [&] { stk_group_norm_kernel<float><<<a.T, 256, lds, as_stream(stream)>>>(a); });
+  else launch_checked("stack norm", [&] { stk_group_norm_kernel<uint16_t><<<a.T, 256, lds, as_stream(stream)>>>(a); });
+}
+
+void vra_stack_moe_sort(const int* pair_expert, const float* pair_weight, int P, int top, int n_groups, int granule, int max_rows, int* row_token,
+                        float* row_scale, int* row_pair, int* tile_group, int64_t stream) {
+  VRA_CHECK_ARG(pair_expert && pair_weight && row_token && row_scale && row_pair && tile_group && P > 0 && top > 0, "stack moe sort: null pointer");
+  VRA_CHECK_ARG((granule == 16 || granule == 64) && max_rows % granule == 0 && max_rows >= P + n_groups * (granule - 1), "stack moe sort: row space too small");
+  const size_t lds = (size_t)n_groups * 3 * sizeof(int);
+  VRA_CHECK_ARG(lds <= 48 * 1024, "stack moe sort: too many experts");
+  launch_checked("stack moe sort", [&] {
+    stk_moe_sort_kernel<<<1, 1024, lds, as_stream(stream)>>>(pair_expert, pair_weight, P, top, n_groups, granule, max_rows, row_token, row_scale, row_pair, tile_group);
+  });
+}
+
+void vra_stack_gated_act(const float* gu, void* out, int M, int F, float limit, float act_alpha, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(gu && out && M > 0 && F > 0, "stack gated act: null pointer or empty shape");
+  if (dtype == VRA_F32) launch_checked("stack gated act", [&] { stk_gated_act_kernel<float><<<M, 256, 0, as_stream(stream)>>>(gu, (float*)out, F, limit, act_alpha); });
+  else launch_checked("stack gated act", [&] { stk_gated_act_kernel<uint16_t><<<M, 256, 0, as_stream(stream)>>>(gu, (uint16_t*)out, F, limit, act_alpha); });
+}
+
+void vra_stack_polynorm(const float* z, void* out, const float* coef, int M, int F, float eps, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(z && out && coef && M > 0 && F > 0, "stack polynorm: null pointer or empty shape");
+  if (dtype == VRA_F32) launch_checked("stack polynorm", [&] { stk_polynorm_kernel<float><<<M, 256, 0, as_stream(stream)>>>(z, (float*)out, coef, F, eps); });
+  else launch_checked("stack polynorm", [&] { stk_polynorm_kernel<uint16_t><<<M, 256, 0, as_stream(stream)>>>(z, (uint16_t*)out, coef, F, eps); });
+}
+
+void vra_stack_residual_combine(float* x, const float* o, const float* p1, int n1, const float* p2, const float* gate, float mult, int T, int W,
+                                int64_t stream) {
+  VRA_CHECK_ARG(x && T > 0 && W > 0 && (n1 == 0 || p1), "stack combine: null pointer or empty shape");
+  launch_checked("stack combine", [&] { stk_residual_combine_kernel<<<T, 256, 0, as_stream(stream)>>>(x, o, p1, n1, p2, gate, mult, W); });
+}
+
+void vra_stack_gather_rows_f32(const float* src, const uint32_t* rows, float* dst, int n, int W, int64_t stream) {
+  VRA_CHECK_ARG(src && rows && dst && n > 0 && W > 0, "stack gather: null pointer or empty shape");
+  launch_checked("stack gather", [&] { stk_gather_rows_kernel<<<n, 256, 0, as_stream(stream)>>>(src, rows, dst, W); });
+}
+
+void vra_stack_kv_store(const void* k, const void* v, int ld, void* kc, void* vc, const int64_t* slots, int T, int kdim, int vdim, int dtype,
+                        int64_t stream) {
+  VRA_CHECK_ARG(k && v && kc && vc && slots && T > 0, "stack kv store: null pointer or empty shape");
+  if (dtype == VRA_F32)
+    launch_checked("stack kv store", [&] { stk_kv_store_kernel<float><<<T, 256, 0, as_stream(stream)>>>((const float*)k, (const float*)v, ld, (float*)kc, (float*)vc, slots, kdim, vdim); });
+  else
+    launch_checked("stack kv store", [&] {
+      stk_kv_store_kernel<uint16_t><<<T, 256, 0, as_stream(stream)>>>((const uint16_t*)k, (const uint16_t*)v, ld, (uint16_t*)kc, (uint16_t*)vc, slots, kdim, vdim);
+    });
+}
+
+void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.q && a.out && a.kc && a.vc && a.positions && a.block_tables && a.context_lens, "stack attention: null pointer");
+  VRA_CHECK_ARG(a.B > 0 && a.H > 0 && a.G > 0 && a.H % a.G == 0 && a.dim > 0 && a.vdim > 0 && a.vdim <= 256 && a.BS > 0 && a.max_blocks > 0,
+                "stack attention: heads must be a multiple of kv heads, value size at most 256");
+  hipStream_t st = as_stream(stream);
+  if (!a.cu_q) {
+    const size_t lds = ((size_t)a.dim + 4 * 64 + 8 + 4 * (size_t)a.vdim) * sizeof(float);
+    VRA_CHECK_ARG(lds <= 64 * 1024, "stack attention: head does not fit LDS");
+    dim3 grid(a.B, a.H);
+    if (dtype == VRA_F32) launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<float><<<grid, 256, lds, st>>>(a); });
+    else launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<uint16_t><<<grid, 256, lds, st>>>(a); });
+    return;
+  }
+  auto need = [&](int kt) { return ((size_t)STK_QT * a.dim + (size_t)kt * (a.dim + 1) + (size_t)kt * a.vdim + (size_t)STK_QT * kt) * sizeof(float); };
+  dim3 grid((a.max_q + STK_QT - 1) / STK_QT, a.B, a.H);
+  const int kt = need(64) <= 64 * 1024 ? 64 : (need(32) <= 64 * 1024 ? 32 : 16);
+  VRA_CHECK_ARG(need(kt) <= 64 * 1024, "stack attention: head does not fit LDS");
+  const size_t lds = need(kt);
+#define STK_PF(TT, KTV) launch_checked("stack attention (prefill)", [&] { stk_attn_prefill_kernel<TT, KTV><<<grid, 256, lds, st>>>(a); })
+  if (dtype == VRA_F32) {
+    if (kt == 64) STK_PF(float, 64);
+    else if (kt == 32) STK_PF(float, 32);
+    else STK_PF(float, 16);
+  } else {
+    if (kt == 64) STK_PF(uint16_t, 64);
+    else if (kt == 32) STK_PF(uint16_t, 32);
+    else STK_PF(uint16_t, 16);
+  }
+#undef STK_PF
+}

@@ -17,6 +17,11 @@ def model_config(cfg):
     """dict with HF config.json-style keys -> ModelConfig (config.rs:218-255)."""
     rs = cfg.get("rope_scaling") or {}
     head_dim = cfg.get("head_dim") or cfg["hidden_size"] // cfg["num_heads"]
+    if cfg.get("arch") in ("stack", 3):  # a list of layers (checkpoint.STACK_ARCHS): the struct carries the sizes, cfg["spec"] the layers
+        return ModelConfig(arch=3, hidden_size=cfg["hidden_size"], intermediate_size=0, num_layers=cfg["num_layers"], num_heads=cfg["num_heads"],
+                           num_kv_heads=cfg["num_kv_heads"], head_dim=cfg["head_dim"], vocab_size=cfg["vocab_size"],
+                           max_position_embeddings=cfg["max_position_embeddings"], rms_norm_eps=cfg["rms_norm_eps"], rope_theta=10000.0,
+                           quant_method=0, bits=16, group_size=0, dtype=cfg.get("dtype", BF16))
     return ModelConfig(
         arch={"llama": 0, 0: 0, "qwen2": 1, 1: 1, "qwen3": 2, 2: 2}[cfg.get("arch", "llama")],
         qk_norm={None: 0, 0: 0, False: 0, "head": 1, 1: 1, True: 1, "full": 2, 2: 2}[cfg.get("qk_norm", 1 if cfg.get("arch") in ("qwen3", 2) else 0)],
@@ -84,7 +89,12 @@ class Engine:
                                use_graph=int(use_graph), tp_rank=tp_rank, tp_world_size=tp_world_size, device=device,
                                seed=seed, fp8_kvcache=int(fp8_kvcache), cpu_mem_fold=cpu_mem_fold,
                                swap_cooling_ms=swap_cooling_ms, min_tokens_left_for_swap=min_tokens_left_for_swap)
-        self.h = self.L.vra_engine_create(C.byref(self.mc), C.byref(self.ec))
+        if self.mc.arch == 3:
+            if max_model_len > 0:  # a layer stack has no position table: the longest sequence is what the engine is asked to hold
+                self.mc.max_position_embeddings = max_model_len
+            self.h = self.L.vra_engine_create_spec(C.byref(self.mc), C.byref(self.ec), cfg["spec"].encode())
+        else:
+            self.h = self.L.vra_engine_create(C.byref(self.mc), C.byref(self.ec))
         if not self.h:
             raise RuntimeError("vra_engine_create failed")
         if comm is not None:
@@ -230,6 +240,36 @@ class Engine:
                                            cu.ctypes.data_as(C.c_void_p) if cu is not None else None, B,
                                            out.ctypes.data_as(C.c_void_p))
         self._check(rc, "forward_raw")
+        return out
+
+    def replay_step(self, entries, end=()):
+        """One step of a replayed trace.  entries: [(request id, tokens, want)] — the request's NEXT tokens and the indices among them
+        whose logits are wanted; all entries run as one batch (portions of prompts beside single decoded tokens).  end: requests that
+        are finished after this step (their pages go back to the block manager).  -> f32 [total wanted, vocab] in entry / want order."""
+        n = len(entries)
+        req = np.ascontiguousarray([e[0] for e in entries], np.int64)
+        counts = np.ascontiguousarray([len(e[1]) for e in entries], np.int32)
+        toks = np.ascontiguousarray([t for e in entries for t in e[1]], np.uint32)
+        n_want = np.ascontiguousarray([len(e[2]) for e in entries], np.int32)
+        want = np.ascontiguousarray([w for e in entries for w in e[2]], np.int32)
+        endv = np.ascontiguousarray(list(end), np.int64)
+        out = np.empty((int(n_want.sum()), self.mc.vocab_size), np.float32)
+        ptr = lambda a: a.ctypes.data_as(C.c_void_p) if a.size else None
+        rc = self.L.vra_engine_replay_step(self.h, n, ptr(req), ptr(counts), ptr(toks), ptr(n_want), ptr(want), len(endv), ptr(endv), ptr(out))
+        self._check(rc, "replay_step")
+        return out
+
+    def layer_trace(self, on=True):
+        """parity instrumentation of layer-stack models: keep the residual stream after every layer run of each forward"""
+        self.L.vra_engine_debug_layer_trace(self.h, int(on))
+        return self
+
+    def read_layer_trace(self, n_tokens):
+        """f32 [layer runs, n_tokens, width] of the last forward (n_tokens = tokens of that step)"""
+        out = np.empty((self.mc.num_layers, n_tokens, self.mc.hidden_size), np.float32)
+        n = self.L.vra_engine_debug_read_layer_trace(self.h, out.ctypes.data_as(C.c_void_p), out.nbytes)
+        if n != out.nbytes:
+            raise RuntimeError("read_layer_trace: the model class keeps no layer trace, or the step had another size")
         return out
 
     TP_STAGES = ("q", "k", "v", "attn", "o_partial", "h_after_o", "act", "down_partial", "h_after_down")

@@ -82,7 +82,8 @@ struct RequestResult {
 
 class Engine {
  public:
-  Engine(const vra_model_config& mc, const vra_engine_config& ec) : mc_(mc), ec_(ec), model_(mc, ec) {
+  Engine(const vra_model_config& mc, const vra_engine_config& ec, const char* spec = nullptr) : mc_(mc), ec_(ec) {
+    model_ = make_model(mc, ec, spec, &error);  // the model class of this architecture (model_base.h)
     if (ec_.block_size <= 0) ec_.block_size = 64;
     if (ec_.prefill_chunk <= 0) ec_.prefill_chunk = 8192;
     // the staging buffers and activations hold kMaxStepTokens rows: a larger chunk is clamped HERE so that the scheduler
@@ -110,10 +111,11 @@ class Engine {
   std::string error;
   vra_model_config mc_;
   vra_engine_config ec_;
-  Model model_;
+  std::unique_ptr<ModelBase> model_;
   std::unique_ptr<BlockManager> bm_;
   std::unique_ptr<Scheduler> sched_;
   std::map<int64_t, RequestResult> results_;
+  std::map<int64_t, Sequence> replay_;  // live requests of a replayed trace (vra_engine_replay_step)
   hipStream_t stream_ = nullptr;
   void* comm_ = nullptr;
   int max_seqs_ = 0, max_model_len_ = 0, max_blocks_per_seq_ = 0, max_step_tokens_ = 0;
@@ -122,7 +124,7 @@ class Engine {
   uint8_t* h_meta_ = nullptr;
   uint8_t* d_meta_ = nullptr;
   size_t meta_bytes_ = 0;
-  size_t off_ids_, off_pos_, off_slots_, off_bt_, off_ctx_, off_cuq_, off_last_, off_dids_, off_dpos_, off_dslots_;
+  size_t off_ids_, off_pos_, off_slots_, off_bt_, off_ctx_, off_cuq_, off_last_, off_dids_, off_dpos_, off_dslots_, off_rows_;
   uint32_t* d_tokens_ = nullptr;
   uint32_t* h_tokens_ = nullptr;
   uint32_t* h_err_ = nullptr;  // pinned copy of the device error words (split-K exchange, one-shot all-reduce), read every step
@@ -164,14 +166,14 @@ class Engine {
       if (dry() || op.pairs.empty()) continue;
       std::vector<int64_t> pairs;
       for (auto& pr : op.pairs) pairs.push_back(pr.first), pairs.push_back(pr.second);
-      const int64_t bb = (int64_t)model_.kv_block_bytes();
-      for (int l = 0; l < mc_.num_layers; l++) {
+      for (int l = 0; l < model_->kv_layers(); l++) {
+        const int64_t kb = (int64_t)model_->k_block_bytes(l), vb = (int64_t)model_->v_block_bytes(l);
         if (op.to_gpu) {
-          vra_swap_blocks(h_swap_k_[l], model_.k_cache(l), pairs.data(), (int)op.pairs.size(), bb, 2, (int64_t)stream_);
-          vra_swap_blocks(h_swap_v_[l], model_.v_cache(l), pairs.data(), (int)op.pairs.size(), bb, 2, (int64_t)stream_);
+          vra_swap_blocks(h_swap_k_[l], model_->k_cache(l), pairs.data(), (int)op.pairs.size(), kb, 2, (int64_t)stream_);
+          vra_swap_blocks(h_swap_v_[l], model_->v_cache(l), pairs.data(), (int)op.pairs.size(), vb, 2, (int64_t)stream_);
         } else {
-          vra_swap_blocks(model_.k_cache(l), h_swap_k_[l], pairs.data(), (int)op.pairs.size(), bb, 1, (int64_t)stream_);
-          vra_swap_blocks(model_.v_cache(l), h_swap_v_[l], pairs.data(), (int)op.pairs.size(), bb, 1, (int64_t)stream_);
+          vra_swap_blocks(model_->k_cache(l), h_swap_k_[l], pairs.data(), (int)op.pairs.size(), kb, 1, (int64_t)stream_);
+          vra_swap_blocks(model_->v_cache(l), h_swap_v_[l], pairs.data(), (int)op.pairs.size(), vb, 1, (int64_t)stream_);
         }
       }
       const char* e = vra_last_error();
@@ -234,6 +236,7 @@ class Engine {
     off_ids_ = o, o += al(T * 4);
     off_pos_ = o, o += al(T * 8);
     off_slots_ = o, o += al(T * 8);
+    off_rows_ = o, o += al(T * 4);  // explicit logit rows of a replayed step (InputMetadata::logit_rows)
     meta_bytes_ = o;
   }
 
@@ -251,32 +254,35 @@ class Engine {
     max_seqs_ = std::max(ec_.max_num_seqs > 0 ? ec_.max_num_seqs : 32, kMinScheduledReqs);
     max_step_tokens_ = kMaxStepTokens;  // a prefill step batches prompts up to this many tokens (1.2 GB of activations for Llama-3-8B)
     // reserve activations first, then give kv_fraction of what is left to the cache
-    if (!model_.init_buffers(std::max(max_step_tokens_, max_seqs_), max_seqs_)) return fail("activation buffers: " + model_.error);
+    if (!model_->init_buffers(std::max(max_step_tokens_, max_seqs_), max_seqs_)) return fail("activation buffers: " + model_->error);
     size_t free_b = 0, total_b = 0;
     (void)hipMemGetInfo(&free_b, &total_b);
-    planned_blocks_ = vra_kv_plan_num_blocks(&mc_, &ec_, (int64_t)free_b);
+    {  // plan_allocation (kvcache_allocator.rs:616-707) with the block size of THIS model class
+      const double frac = ec_.kv_fraction > 0 ? ec_.kv_fraction : (ec_.max_model_len > 0 ? 0.95 : 0.5);
+      const int64_t per = model_->kv_bytes_per_block();
+      planned_blocks_ = ec_.num_gpu_blocks > 0 ? ec_.num_gpu_blocks : (per > 0 ? (int64_t)((double)free_b * frac) / per : 0);
+    }
     if (planned_blocks_ > (1 << 24)) planned_blocks_ = 1 << 24;
     prepared_ = true;
     return true;
   }
   bool finalize() {
     if (dry()) return finalize_dry();
-    if (model_.world() > 1 && !model_.has_comm()) return fail("tensor parallel world_size > 1 without a communicator (vra_engine_set_comm before finalize)");
-    if (model_.world() > 1 && ec_.num_gpu_blocks <= 0)
+    if (model_->world() > 1 && !model_->has_comm()) return fail("tensor parallel world_size > 1 without a communicator (vra_engine_set_comm before finalize)");
+    if (model_->world() > 1 && ec_.num_gpu_blocks <= 0)
       return fail("tensor parallel: num_gpu_blocks must be set explicitly and identically on every rank (vra_engine_plan_kv_blocks on each rank, take the minimum, vra_engine_set_num_gpu_blocks)");
     if (!prepare()) return false;
     int64_t nb = ec_.num_gpu_blocks > 0 ? ec_.num_gpu_blocks : planned_blocks_;
     if (nb < 2) return fail("not enough memory for the KV cache");
     if (nb > (1 << 24)) nb = 1 << 24;
-    if (!model_.init_kv_cache((int)nb)) return fail("kv cache: " + model_.error);
+    if (!model_->init_kv_cache((int)nb)) return fail("kv cache: " + model_->error);
     setup_host(nb);
     if (num_cpu_blocks_ > 0) {  // pinned host copies of whole blocks, per layer: K then V (kvcache_allocator.rs:905-930)
-      const size_t bytes = (size_t)num_cpu_blocks_ * model_.kv_block_bytes();
-      h_swap_k_.assign(mc_.num_layers, nullptr);
-      h_swap_v_.assign(mc_.num_layers, nullptr);
-      for (int l = 0; l < mc_.num_layers; l++)
-        if (hipHostMalloc(&h_swap_k_[l], bytes, hipHostMallocDefault) != hipSuccess ||
-            hipHostMalloc(&h_swap_v_[l], bytes, hipHostMallocDefault) != hipSuccess)
+      h_swap_k_.assign(model_->kv_layers(), nullptr);
+      h_swap_v_.assign(model_->kv_layers(), nullptr);
+      for (int l = 0; l < model_->kv_layers(); l++)
+        if (hipHostMalloc(&h_swap_k_[l], (size_t)num_cpu_blocks_ * model_->k_block_bytes(l), hipHostMallocDefault) != hipSuccess ||
+            hipHostMalloc(&h_swap_v_[l], (size_t)num_cpu_blocks_ * model_->v_block_bytes(l), hipHostMallocDefault) != hipSuccess)
           return fail("pinned alloc for the CPU swap space failed");
     }
     const size_t B = max_seqs_;
@@ -290,13 +296,19 @@ class Engine {
     if (hipMalloc((void**)&d_pen_, pen_bytes) != hipSuccess) return fail("penalty staging alloc failed");
     memset(h_meta_, 0, meta_bytes_);
     memset(h_err_, 0, 64);
-    if (ec_.use_graph && !warmup_capture()) return false;
+    if (ec_.use_graph && model_->graph_capturable() && !warmup_capture()) return false;
     return true;
   }
 
   // ---- ModelRunner::prepare_prefill (runner.rs:978-1241)
   InputMetadata prepare_prefill(const std::vector<int>& ids, int* n_copy_bytes) {
     auto& run = sched_->running();
+    std::vector<const Sequence*> seqs;
+    for (int id : ids) seqs.push_back(&run[id]);
+    return prepare_prefill_seqs(seqs, n_copy_bytes);
+  }
+  // the same over any live sequences (the scheduler's running list, or the requests of a replayed trace)
+  InputMetadata prepare_prefill_seqs(const std::vector<const Sequence*>& seqs, int* n_copy_bytes) {
     uint32_t* h_ids = (uint32_t*)(h_meta_ + off_ids_);
     int64_t* h_pos = (int64_t*)(h_meta_ + off_pos_);
     int64_t* h_slots = (int64_t*)(h_meta_ + off_slots_);
@@ -309,16 +321,16 @@ class Engine {
     InputMetadata md;
     {  // the token count is checked BEFORE anything is written to the staging buffers
       int64_t total = 0;
-      for (int id : ids) total += std::min(CHUNK, run[id].len() - run[id].num_cached_tokens);
-      if (total > std::max(max_step_tokens_, max_seqs_) || (int)ids.size() > max_seqs_) {
+      for (const Sequence* sp : seqs) total += std::min(CHUNK, sp->len() - sp->num_cached_tokens);
+      if (total > std::max(max_step_tokens_, max_seqs_) || (int)seqs.size() > max_seqs_) {
         md.n_tokens = -1;
         return md;
       }
     }
-    for (int id : ids) max_bt = std::max(max_bt, (int)run[id].block_table.size());
+    for (const Sequence* sp : seqs) max_bt = std::max(max_bt, (int)sp->block_table.size());
     h_cuq[0] = 0;
-    for (size_t b = 0; b < ids.size(); b++) {
-      const Sequence& s = run[ids[b]];
+    for (size_t b = 0; b < seqs.size(); b++) {
+      const Sequence& s = *seqs[b];
       const int n = std::min(CHUNK, s.len() - s.num_cached_tokens);
       for (int i = 0; i < n; i++) {
         h_ids[T + i] = s.token_ids[s.num_cached_tokens + i];
@@ -348,7 +360,7 @@ class Engine {
     }
     md.is_prefill = true;
     md.n_tokens = T;
-    md.n_seqs = (int)ids.size();
+    md.n_seqs = (int)seqs.size();
     md.max_blocks = max_bt;
     md.max_seqlen_q = max_q;
     md.max_context_len = max_ctx;
@@ -407,6 +419,7 @@ class Engine {
   bool upload_meta(const InputMetadata& md) {
     size_t bytes = off_bt_ + (size_t)md.n_seqs * (md.is_prefill ? md.max_blocks : max_blocks_per_seq_) * 4;
     if (md.is_prefill) bytes = off_slots_ + (size_t)md.n_tokens * 8;
+    if (md.n_logit_rows > 0) bytes = off_rows_ + (size_t)md.n_logit_rows * 4;
     bytes = std::min(meta_bytes_, (bytes + 255) & ~(size_t)255);
     return hipMemcpyAsync(d_meta_, h_meta_, bytes, hipMemcpyHostToDevice, stream_) == hipSuccess;
   }
@@ -444,12 +457,12 @@ class Engine {
     hipGraph_t g = nullptr;
     hipGraphExec_t ge = nullptr;
     if (hipStreamBeginCapture(stream_, hipStreamCaptureModeRelaxed) != hipSuccess) return nullptr;
-    const bool ok = model_.forward(cmd, (int64_t)stream_, d_tokens_);
+    const bool ok = model_->forward(cmd, (int64_t)stream_, d_tokens_);
     const hipError_t e = hipStreamEndCapture(stream_, &g);
     if (ok && e == hipSuccess && g && hipGraphInstantiate(&ge, g, nullptr, nullptr, 0) == hipSuccess) graphs_[key] = ge;
     else ge = nullptr;
     if (g) (void)hipGraphDestroy(g);
-    if (!ok) fail("graph capture: " + model_.error);
+    if (!ok) fail("graph capture: " + model_->error);
     return ge;
   }
   // warmup_capture (engine.rs:108-503 → graph.rs:448-560): all decode graphs are captured at init, so that no request
@@ -477,7 +490,7 @@ class Engine {
       if (!upload_meta(md)) return fail("metadata upload failed");
       last_graph_ = nullptr;  // (vra_engine_bench_replay replays the decode graph of the MOST RECENT step only: ADVICE r4)
       RoctxRange range("prefill", md.n_tokens, B);
-      if (!model_.forward(md, (int64_t)stream_, d_tokens_)) return fail(model_.error);
+      if (!model_->forward(md, (int64_t)stream_, d_tokens_)) return fail(model_->error);
     } else {
       const int bucket = std::min(batch_bucket(B), max_seqs_);
       InputMetadata md = prepare_decode(ids, std::max(bucket, B));
@@ -496,7 +509,7 @@ class Engine {
       }
       if (!launched) {
         last_graph_ = nullptr;
-        if (!model_.forward(md, (int64_t)stream_, d_tokens_)) return fail(model_.error);
+        if (!model_->forward(md, (int64_t)stream_, d_tokens_)) return fail(model_->error);
       }
     }
     if (!sample_stochastic(ids, is_prefill)) return false;
@@ -569,17 +582,17 @@ class Engine {
         const size_t bytes = (size_t)max_seqs_ * (kPenaltyWindow * 4 + 12);
         if (hipMemcpyAsync(d_pen_, h_pen_ctx_, bytes, hipMemcpyHostToDevice, stream_) != hipSuccess) return fail("penalty upload failed");
         const uint8_t* d_len = d_pen_ + (size_t)max_seqs_ * kPenaltyWindow * 4;
-        vra_apply_penalties(model_.logits(), (const uint32_t*)d_pen_, (const int32_t*)d_len, B, kPenaltyWindow, mc_.vocab_size,
+        vra_apply_penalties(model_->logits(), (const uint32_t*)d_pen_, (const int32_t*)d_len, B, kPenaltyWindow, mc_.vocab_size,
                             (const float*)(d_len + (size_t)max_seqs_ * 4), (const float*)(d_len + (size_t)max_seqs_ * 8), (int64_t)stream_);
       }
     }
     if (c.kind == 0) {  // greedy with penalties
-      vra_argmax_f32(model_.logits(), d_tokens_, B, mc_.vocab_size, (int64_t)stream_);
+      vra_argmax_f32(model_->logits(), d_tokens_, B, mc_.vocab_size, (int64_t)stream_);
     } else {
       // one fresh seed per call, as `self.rng.lock().next_u64()` (logits_processor.rs:223-226)
       ++sample_calls_;
       const uint64_t seed = (uint64_t)vra_hash32_host(ec_.seed ? ec_.seed : 1234, sample_calls_) << 32 | vra_hash32_host(ec_.seed + 1, sample_calls_);
-      vra_sample(model_.logits(), d_tokens_, B, mc_.vocab_size, c.k, c.p, c.temperature, seed, nullptr, nullptr, (int64_t)stream_);
+      vra_sample(model_->logits(), d_tokens_, B, mc_.vocab_size, c.k, c.p, c.temperature, seed, nullptr, nullptr, (int64_t)stream_);
     }
     const char* e = vra_last_error();
     if (e && e[0]) return fail(std::string("sampler: ") + e);
@@ -775,22 +788,39 @@ extern "C" int32_t vra_pc_evict_blocks(void* pc, int32_t n, int32_t* h_evicted, 
 extern "C" void* vra_engine_create(const vra_model_config* mc, const vra_engine_config* ec) {
   if (!mc || !ec) return nullptr;
   if (ec->device >= 0 && hipSetDevice(ec->device) != hipSuccess) return nullptr;
-  return new Engine(*mc, *ec);
+  Engine* en = new Engine(*mc, *ec);
+  if (!en->model_) {
+    delete en;
+    return nullptr;
+  }
+  return en;
+}
+// the same for architectures whose layers are listed one by one (VRA_ARCH_STACK; host/stack_model.h gives the text's format).  A spec
+// that does not parse leaves an engine whose first call fails with the reason (vra_engine_last_error).
+extern "C" void* vra_engine_create_spec(const vra_model_config* mc, const vra_engine_config* ec, const char* spec) {
+  if (!mc || !ec) return nullptr;
+  if (ec->device >= 0 && hipSetDevice(ec->device) != hipSuccess) return nullptr;
+  Engine* en = new Engine(*mc, *ec, spec);
+  if (!en->model_) {
+    delete en;
+    return nullptr;
+  }
+  return en;
 }
 extern "C" void vra_engine_destroy(void* e) { delete static_cast<Engine*>(e); }
 extern "C" const char* vra_engine_last_error(const void* e) { return static_cast<const Engine*>(e)->error.c_str(); }
 extern "C" int32_t vra_engine_init_synthetic(void* e) {
   auto* en = static_cast<Engine*>(e);
-  if (!en->model_.init_synthetic(en->ec_.seed ? en->ec_.seed : 1234)) {
-    en->error = en->model_.error;
+  if (!en->model_->init_synthetic(en->ec_.seed ? en->ec_.seed : 1234)) {
+    en->error = en->model_->error;
     return -1;
   }
   return 0;
 }
 extern "C" int32_t vra_engine_load_tensor(void* e, const char* name, const void* h_data, const int64_t* shape, int32_t ndim, int32_t elem_bytes) {
   auto* en = static_cast<Engine*>(e);
-  if (!en->model_.load_tensor(name, h_data, shape, ndim, elem_bytes)) {
-    en->error = en->model_.error;
+  if (!en->model_->load_tensor(name, h_data, shape, ndim, elem_bytes)) {
+    en->error = en->model_->error;
     return -1;
   }
   return 0;
@@ -798,14 +828,14 @@ extern "C" int32_t vra_engine_load_tensor(void* e, const char* name, const void*
 extern "C" int32_t vra_engine_set_comm(void* e, void* comm) {
   auto* en = static_cast<Engine*>(e);
   en->comm_ = comm;
-  en->model_.set_comm(comm);
+  en->model_->set_comm(comm);
   return 0;
 }
 extern "C" int32_t vra_engine_finalize_weights(void* e) {
   auto* en = static_cast<Engine*>(e);
   if (en->dry()) return en->finalize() ? 0 : -1;
-  if (!en->model_.finalize_weights()) {  // repack of explicit tensors; a no-op after synthetic init (idempotent)
-    en->error = en->model_.error;
+  if (!en->model_->finalize_weights()) {  // repack of explicit tensors; a no-op after synthetic init (idempotent)
+    en->error = en->model_->error;
     return -1;
   }
   return en->finalize() ? 0 : -1;
@@ -816,7 +846,7 @@ extern "C" int32_t vra_engine_copy_logits(void* e, float* h_out, int32_t n_seqs)
     en->error = "vra_engine_copy_logits: finalised GPU engine and 1..max_num_seqs rows";
     return -1;
   }
-  if (hipMemcpyAsync(h_out, en->model_.logits(), (size_t)n_seqs * en->mc_.vocab_size * 4, hipMemcpyDeviceToHost, en->stream_) != hipSuccess ||
+  if (hipMemcpyAsync(h_out, en->model_->logits(), (size_t)n_seqs * en->mc_.vocab_size * 4, hipMemcpyDeviceToHost, en->stream_) != hipSuccess ||
       hipStreamSynchronize(en->stream_) != hipSuccess) {
     en->error = "vra_engine_copy_logits: copy failed";
     return -1;
@@ -827,20 +857,20 @@ extern "C" int32_t vra_engine_copy_logits(void* e, float* h_out, int32_t n_seqs)
 // the engine so that the oracle restates the order the engine actually runs
 extern "C" int32_t vra_engine_norm_deferred(void* e, int32_t rows, int32_t layer) {
   auto* en = static_cast<Engine*>(e);
-  return en->dry() ? 0 : en->model_.norm_deferred_mask(rows, layer);
+  return en->dry() ? 0 : en->model_->norm_deferred_mask(rows, layer);
 }
 // parity instrumentation of the tensor-parallel forward (model.h `set_tp_snapshots`): stage copies of one layer (`on` = 1 + the layer, 0 = off), read back per stage
-extern "C" void vra_engine_debug_tp_snapshots(void* e, int32_t on) { static_cast<Engine*>(e)->model_.set_tp_snapshots(on); }
+extern "C" void vra_engine_debug_tp_snapshots(void* e, int32_t on) { static_cast<Engine*>(e)->model_->set_tp_snapshots(on); }
 extern "C" int64_t vra_engine_debug_read_tp_snapshot(void* e, int32_t idx, void* h_out, int64_t max_bytes) {
   auto* en = static_cast<Engine*>(e);
   if (en->dry()) return -1;
-  return en->model_.read_tp_snapshot(idx, h_out, max_bytes, (int64_t)en->stream_);
+  return en->model_->read_tp_snapshot(idx, h_out, max_bytes, (int64_t)en->stream_);
 }
 extern "C" int32_t vra_engine_finalize_model(void* e) {
   auto* en = static_cast<Engine*>(e);
   if (en->dry()) return 0;
-  if (!en->model_.finalize_weights()) {
-    en->error = en->model_.error;
+  if (!en->model_->finalize_weights()) {
+    en->error = en->model_->error;
     return -1;
   }
   return 0;
@@ -864,8 +894,8 @@ extern "C" int32_t vra_engine_update_config(void* e, const vra_engine_config* cf
 extern "C" int64_t vra_engine_plan_kv_blocks(void* e) {
   auto* en = static_cast<Engine*>(e);
   if (en->dry()) return en->ec_.num_gpu_blocks;
-  if (!en->model_.finalize_weights()) {
-    en->error = en->model_.error;
+  if (!en->model_->finalize_weights()) {
+    en->error = en->model_->error;
     return -1;
   }
   if (!en->prepare()) return -1;
@@ -889,7 +919,7 @@ extern "C" int32_t vra_engine_swap_blocks(void* e, const int64_t* h_pairs, int32
     en->error = "vra_engine_swap_blocks: no CPU swap space (vra_engine_config.cpu_mem_fold = 0, or a host-only engine)";
     return -1;
   }
-  const int64_t ngpu = en->model_.num_blocks(), ncpu = en->num_cpu_blocks_;
+  const int64_t ngpu = en->model_->num_blocks(), ncpu = en->num_cpu_blocks_;
   for (int i = 0; i < n_pairs; i++) {
     const int64_t src = h_pairs[2 * i], dst = h_pairs[2 * i + 1];
     if (src < 0 || dst < 0 || src >= (swap_in ? ncpu : ngpu) || dst >= (swap_in ? ngpu : ncpu)) {
@@ -897,14 +927,14 @@ extern "C" int32_t vra_engine_swap_blocks(void* e, const int64_t* h_pairs, int32
       return -1;
     }
   }
-  const int64_t bb = (int64_t)en->model_.kv_block_bytes();
-  for (int l = 0; l < en->mc_.num_layers; l++) {
+  for (int l = 0; l < en->model_->kv_layers(); l++) {
+    const int64_t kb = (int64_t)en->model_->k_block_bytes(l), vb = (int64_t)en->model_->v_block_bytes(l);
     if (swap_in) {
-      vra_swap_blocks(en->h_swap_k_[l], en->model_.k_cache(l), h_pairs, n_pairs, bb, 2, (int64_t)en->stream_);
-      vra_swap_blocks(en->h_swap_v_[l], en->model_.v_cache(l), h_pairs, n_pairs, bb, 2, (int64_t)en->stream_);
+      vra_swap_blocks(en->h_swap_k_[l], en->model_->k_cache(l), h_pairs, n_pairs, kb, 2, (int64_t)en->stream_);
+      vra_swap_blocks(en->h_swap_v_[l], en->model_->v_cache(l), h_pairs, n_pairs, vb, 2, (int64_t)en->stream_);
     } else {
-      vra_swap_blocks(en->model_.k_cache(l), en->h_swap_k_[l], h_pairs, n_pairs, bb, 1, (int64_t)en->stream_);
-      vra_swap_blocks(en->model_.v_cache(l), en->h_swap_v_[l], h_pairs, n_pairs, bb, 1, (int64_t)en->stream_);
+      vra_swap_blocks(en->model_->k_cache(l), en->h_swap_k_[l], h_pairs, n_pairs, kb, 1, (int64_t)en->stream_);
+      vra_swap_blocks(en->model_->v_cache(l), en->h_swap_v_[l], h_pairs, n_pairs, vb, 1, (int64_t)en->stream_);
     }
   }
   (swap_in ? en->swap_in_blocks_ : en->swap_out_blocks_) += n_pairs;
@@ -922,7 +952,7 @@ extern "C" void vra_engine_swap_stats(const void* e, int64_t* out4) {
   out4[2] = en->swap_out_blocks_;
   out4[3] = en->swap_in_blocks_;
 }
-extern "C" int32_t vra_engine_num_gpu_blocks(const void* e) { return static_cast<const Engine*>(e)->model_.num_blocks(); }
+extern "C" int32_t vra_engine_num_gpu_blocks(const void* e) { return static_cast<const Engine*>(e)->model_->num_blocks(); }
 extern "C" int64_t vra_engine_add_request(void* e, const uint32_t* h_prompt, int32_t n_prompt, int32_t max_tokens, int32_t ignore_eos,
                                           const uint32_t* h_eos, int32_t n_eos) {
   auto* en = static_cast<Engine*>(e);
@@ -1043,7 +1073,7 @@ struct RawSampling {
 static int32_t forward_raw_impl(Engine* en, const uint32_t* h_ids, const int64_t* h_positions, const int64_t* h_slot_mapping,
                                 int32_t n_tokens, int32_t is_prefill, const uint32_t* h_block_tables, int32_t max_blocks,
                                 const uint32_t* h_context_lens, const uint32_t* h_cu_seqlens_q, int32_t n_seqs,
-                                float* h_logits_out, uint32_t* h_tokens_out, const RawSampling* smp) {
+                                float* h_logits_out, uint32_t* h_tokens_out, const RawSampling* smp, const uint32_t* h_rows = nullptr, int32_t n_rows = 0) {
   if (!en->sched_) {
     en->error = "engine not finalised";
     return -1;
@@ -1064,7 +1094,7 @@ static int32_t forward_raw_impl(Engine* en, const uint32_t* h_ids, const int64_t
     return -1;
   }
   {
-    const int64_t n_slots = (int64_t)en->model_.num_blocks() * en->ec_.block_size;
+    const int64_t n_slots = (int64_t)en->model_->num_blocks() * en->ec_.block_size;
     const int64_t max_ctx = (int64_t)max_blocks * en->ec_.block_size;
     for (int t = 0; t < n_tokens; t++) {
       if (h_ids[t] >= (uint32_t)en->mc_.vocab_size) return en->error = "forward_raw: token id " + std::to_string(h_ids[t]) + " outside the vocabulary", -1;
@@ -1078,7 +1108,7 @@ static int32_t forward_raw_impl(Engine* en, const uint32_t* h_ids, const int64_t
       if ((int64_t)h_context_lens[b] > max_ctx) return en->error = "forward_raw: context length beyond the block table", -1;
       const int used = (int)(((int64_t)h_context_lens[b] + en->ec_.block_size - 1) / en->ec_.block_size);
       for (int k = 0; k < used; k++)
-        if (h_block_tables[(size_t)b * max_blocks + k] >= (uint32_t)en->model_.num_blocks())
+        if (h_block_tables[(size_t)b * max_blocks + k] >= (uint32_t)en->model_->num_blocks())
           return en->error = "forward_raw: block id " + std::to_string(h_block_tables[(size_t)b * max_blocks + k]) + " outside the KV cache", -1;
     }
     if (is_prefill) {
@@ -1126,6 +1156,14 @@ static int32_t forward_raw_impl(Engine* en, const uint32_t* h_ids, const int64_t
     }
   }
   en->bind(md);
+  if (n_rows > 0) {  // explicit logit rows (replayed traces): any rows of the step, in the caller's order
+    if (!h_rows || n_rows > en->model_->max_logit_rows()) return en->error = "forward_raw: more logit rows than the model's logits buffer holds", -1;
+    for (int i = 0; i < n_rows; i++)
+      if (h_rows[i] >= (uint32_t)n_tokens) return en->error = "forward_raw: logit row outside the step", -1;
+    memcpy(en->h_meta_ + en->off_rows_, h_rows, (size_t)n_rows * 4);
+    md.logit_rows = (const uint32_t*)(en->d_meta_ + en->off_rows_);
+    md.n_logit_rows = n_rows;
+  }
   if (!en->upload_meta(md)) return -1;
   bool launched = false;
   if (graph_decode) {
@@ -1136,18 +1174,19 @@ static int32_t forward_raw_impl(Engine* en, const uint32_t* h_ids, const int64_t
       launched = true;
     }
   }
-  if (!launched && !en->model_.forward(md, (int64_t)en->stream_, h_tokens_out ? en->d_tokens_ : nullptr)) {
-    en->error = en->model_.error;
+  if (!launched && !en->model_->forward(md, (int64_t)en->stream_, h_tokens_out ? en->d_tokens_ : nullptr)) {
+    en->error = en->model_->error;
     return -1;
   }
   en->last_graph_ = nullptr;
   if (h_logits_out &&
-      hipMemcpyAsync(h_logits_out, en->model_.logits(), (size_t)n_seqs * en->mc_.vocab_size * 4, hipMemcpyDeviceToHost, en->stream_) != hipSuccess)
+      hipMemcpyAsync(h_logits_out, en->model_->logits(), (size_t)(n_rows > 0 ? n_rows : n_seqs) * en->mc_.vocab_size * 4, hipMemcpyDeviceToHost,
+                     en->stream_) != hipSuccess)
     return -1;
   if (h_tokens_out) {
     if (smp && smp->kind == 1) {  // LogitsProcessor::sample_with_strategy on the device logits (logits_processor.rs:199-271)
       if (smp->k > 256) return en->error = "top_k > 256 is not supported by the device sampler", -1;
-      vra_sample(en->model_.logits(), en->d_tokens_, n_seqs, en->mc_.vocab_size, smp->k, smp->p, smp->t, smp->seed, nullptr, nullptr, (int64_t)en->stream_);
+      vra_sample(en->model_->logits(), en->d_tokens_, n_seqs, en->mc_.vocab_size, smp->k, smp->p, smp->t, smp->seed, nullptr, nullptr, (int64_t)en->stream_);
       const char* se = vra_last_error();
       if (se && se[0]) return en->error = std::string("sampler: ") + se, -1;
     }
@@ -1195,6 +1234,84 @@ extern "C" int32_t vra_engine_forward_tokens(void* e, const uint32_t* h_ids, con
   smp.kind = stochastic ? 1 : 0, smp.k = top_k, smp.p = top_p, smp.t = temperature, smp.seed = seed;
   return forward_raw_impl(static_cast<Engine*>(e), h_ids, h_positions, h_slot_mapping, n_tokens, is_prefill, h_block_tables, max_blocks, h_context_lens,
                           h_cu_seqlens_q, n_seqs, nullptr, h_tokens_out, &smp);
+}
+
+// ---- replayed traces (bin/trace_run): the caller says which tokens of which request run in a step — portions of prompts beside single
+// decoded tokens, all one batch — and at which of them it wants the logits.  A request is admitted at its first entry, keeps its pages in
+// THIS engine's block manager while it is live (it may sit out steps) and hands them back when the caller ends it.  Steps in which every
+// entry brings one token behind a cached context run in the decode form (decode kernels), every other step in the prefill form.
+extern "C" int32_t vra_engine_replay_step(void* e, int32_t n_entries, const int64_t* h_req, const int32_t* h_counts, const uint32_t* h_tokens,
+                                          const int32_t* h_n_want, const int32_t* h_want, int32_t n_end, const int64_t* h_end, float* h_logits_out) {
+  auto* en = static_cast<Engine*>(e);
+  if (en->dry() || !en->sched_) return en->error = "replay_step: finalised GPU engine needed", -1;
+  if (n_entries < 0 || n_entries > en->max_seqs_ || (n_entries > 0 && (!h_req || !h_counts || !h_tokens || !h_n_want)))
+    return en->error = "replay_step: too many entries for max_num_seqs, or null argument", -1;
+  const int BS = en->ec_.block_size;
+  std::vector<vra::Sequence*> seqs;
+  int T = 0, total_want = 0;
+  bool decode = n_entries > 0;
+  for (int i = 0; i < n_entries; i++) {
+    if (h_counts[i] <= 0) return en->error = "replay_step: an entry without tokens", -1;
+    for (int j = 0; j < i; j++)
+      if (h_req[j] == h_req[i]) return en->error = "replay_step: a request appears twice in one step", -1;
+    vra::Sequence& s = en->replay_[h_req[i]];
+    if (s.token_ids.empty()) s.id = h_req[i], s.block_size = BS;
+    if (s.len() + h_counts[i] > en->max_model_len_) return en->error = "replay_step: request longer than max_model_len", -1;
+    decode = decode && h_counts[i] == 1 && s.num_cached_tokens > 0;
+    s.token_ids.insert(s.token_ids.end(), h_tokens + T, h_tokens + T + h_counts[i]);
+    if (!en->bm_->ensure_allocate(s)) return en->error = "replay_step: no free KV block (the pool is smaller than the live requests need)", -1;
+    seqs.push_back(&s);
+    T += h_counts[i];
+    for (int j = 0; j < h_n_want[i]; j++)
+      if (!h_want || h_want[total_want + j] < 0 || h_want[total_want + j] >= h_counts[i]) return en->error = "replay_step: wanted row outside the entry", -1;
+    total_want += h_n_want[i];
+  }
+  if (n_entries > 0) {
+    int max_bt = 1;
+    for (auto* s : seqs) max_bt = std::max(max_bt, (int)s->block_table.size());
+    std::vector<uint32_t> ids(T), bt((size_t)n_entries * max_bt, 0), ctx(n_entries), cu(n_entries + 1, 0), rows;
+    std::vector<int64_t> pos(T), slots(T);
+    int t = 0, w = 0;
+    for (int i = 0; i < n_entries; i++) {
+      const vra::Sequence& s = *seqs[i];
+      for (int p = s.num_cached_tokens; p < s.len(); p++, t++) {
+        ids[t] = s.token_ids[p], pos[t] = p;
+        slots[t] = (int64_t)s.block_table[p / BS] * BS + p % BS;
+      }
+      for (size_t j = 0; j < s.block_table.size(); j++) bt[(size_t)i * max_bt + j] = s.block_table[j];
+      ctx[i] = (uint32_t)s.len();
+      cu[i + 1] = (uint32_t)t;
+      for (int j = 0; j < h_n_want[i]; j++) rows.push_back(cu[i] + (uint32_t)h_want[w + j]);
+      w += h_n_want[i];
+    }
+    if (total_want > 0 && !h_logits_out) return en->error = "replay_step: logits wanted without a buffer", -1;
+    std::vector<float> scratch;
+    float* out = h_logits_out;
+    if (total_want == 0) {  // the step only fills the cache: the forward still answers one row, which nobody reads
+      scratch.resize((size_t)en->mc_.vocab_size);
+      out = scratch.data();
+      rows.assign(1, 0);
+    }
+    if (forward_raw_impl(en, ids.data(), pos.data(), slots.data(), T, decode ? 0 : 1, bt.data(), max_bt, ctx.data(), decode ? nullptr : cu.data(), n_entries, out,
+                         nullptr, nullptr, rows.data(), (int32_t)rows.size()) != 0)
+      return -1;
+    for (auto* s : seqs) s->num_cached_tokens = s->len();
+  }
+  for (int i = 0; i < n_end; i++) {
+    auto it = en->replay_.find(h_end[i]);
+    if (it == en->replay_.end()) continue;
+    en->bm_->deallocate(it->second);
+    en->replay_.erase(it);
+  }
+  return total_want;
+}
+// parity instrumentation of layer stacks: keep the residual stream after every layer run of each forward; read the last forward's copy
+// (f32 [layer runs, tokens of the step, width]); -1 where the model class does not offer it
+extern "C" void vra_engine_debug_layer_trace(void* e, int32_t on) { static_cast<Engine*>(e)->model_->set_layer_trace(on != 0); }
+extern "C" int64_t vra_engine_debug_read_layer_trace(void* e, void* h_out, int64_t max_bytes) {
+  auto* en = static_cast<Engine*>(e);
+  if (en->dry()) return -1;
+  return en->model_->read_layer_trace(h_out, max_bytes, (int64_t)en->stream_);
 }
 
 extern "C" double vra_engine_timed_decode(void* e, int32_t steps) {
@@ -1247,12 +1364,12 @@ extern "C" double vra_engine_bench_gemm(void* e, int32_t which, int32_t m, int32
   auto* en = static_cast<Engine*>(e);
   const int L = en->mc_.num_layers;
   for (int i = 0; i < L; i++)
-    if (!en->model_.launch_gemm(which, i % L, m, (int64_t)en->stream_)) return -1.0;
+    if (!en->model_->launch_gemm(which, i % L, m, (int64_t)en->stream_)) return -1.0;
   hipEvent_t a, b;
   (void)hipEventCreate(&a);
   (void)hipEventCreate(&b);
   (void)hipEventRecord(a, en->stream_);
-  for (int i = 0; i < iters; i++) en->model_.launch_gemm(which, i % L, m, (int64_t)en->stream_);
+  for (int i = 0; i < iters; i++) en->model_->launch_gemm(which, i % L, m, (int64_t)en->stream_);
   (void)hipEventRecord(b, en->stream_);
   (void)hipEventSynchronize(b);
   float ms = 0.f;
@@ -1262,6 +1379,6 @@ extern "C" double vra_engine_bench_gemm(void* e, int32_t which, int32_t m, int32
   return (double)ms / iters;
 }
 extern "C" int64_t vra_engine_gemm_bytes(const void* e, int32_t which, int32_t m) {
-  return static_cast<const Engine*>(e)->model_.gemm_algorithmic_bytes(which, m);
+  return static_cast<const Engine*>(e)->model_->gemm_algorithmic_bytes(which, m);
 }
-extern "C" int64_t vra_engine_weight_bytes(const void* e) { return (int64_t) static_cast<const Engine*>(e)->model_.weight_bytes(); }
+extern "C" int64_t vra_engine_weight_bytes(const void* e) { return (int64_t) static_cast<const Engine*>(e)->model_->weight_bytes(); }

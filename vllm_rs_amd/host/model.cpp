@@ -1135,7 +1135,15 @@ bool Model::forward(const InputMetadata& md, int64_t stream, uint32_t* tokens) {
   // last token of every sequence (llama.rs:306-310), final norm, lm_head -> f32 (llama.rs:311-320)
   const void* xin = h_;
   int rows = T;
-  if (md.is_prefill) {
+  if (md.n_logit_rows > 0) {  // explicit rows (replayed traces): any rows of the step, as many as the logits buffer holds
+    if (md.n_logit_rows > max_seqs_) {
+      error = "forward: more logit rows than max_num_seqs";
+      return false;
+    }
+    vra_index_select_rows(h_, md.logit_rows, last_, md.n_logit_rows, H, dt_, stream);
+    xin = last_;
+    rows = md.n_logit_rows;
+  } else if (md.is_prefill) {
     vra_index_select_rows(h_, md.last_token_rows, last_, B, H, dt_, stream);
     xin = last_;
     rows = B;

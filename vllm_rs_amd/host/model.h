@@ -12,6 +12,7 @@
 #include <vector>
 
 #include "../../include/vllm_rs_amd.h"
+#include "model_base.h"
 
 struct GemvSArgs;  // csrc/gemv_q4s.cuh
 
@@ -47,72 +48,58 @@ struct LayerWeights {
   uint32_t* qkv_z_um = nullptr;
 };
 
-// The data contract between runner and kernels (InputMetadata, runner.rs:1222-1238,1369-1385);
-// all pointers are device buffers owned by the runner.
-struct InputMetadata {
-  bool is_prefill = false;
-  int n_tokens = 0;
-  int n_seqs = 0;
-  const uint32_t* input_ids = nullptr;      // [T]
-  const int64_t* positions = nullptr;       // [T]
-  const int64_t* slot_mapping = nullptr;    // [T]
-  const uint32_t* block_tables = nullptr;   // [B, max_blocks]
-  const uint32_t* context_lens = nullptr;   // [B]
-  const uint32_t* cu_seqlens_q = nullptr;   // [B+1] (prefill)
-  const uint32_t* last_token_rows = nullptr;  // [B] = seqlens[i]-1 (llama.rs:306-310)
-  int max_blocks = 0;
-  int max_seqlen_q = 0;
-  int max_context_len = 0;
-};
-
-class Model {
+class Model : public ModelBase {
  public:
   Model(const vra_model_config& mc, const vra_engine_config& ec);
-  ~Model();
-  std::string error;
+  ~Model() override;
 
   // weights
-  bool init_synthetic(uint64_t seed);
-  bool load_tensor(const std::string& name, const void* host, const int64_t* shape, int ndim, int elem_bytes);
-  bool finalize_weights();   // repack staged checkpoint tensors, check completeness
+  bool init_synthetic(uint64_t seed) override;
+  bool load_tensor(const std::string& name, const void* host, const int64_t* shape, int ndim, int elem_bytes) override;
+  bool finalize_weights() override;   // repack staged checkpoint tensors, check completeness
   // kv cache
-  bool init_kv_cache(int num_blocks);
-  int num_blocks() const { return num_blocks_; }
+  bool init_kv_cache(int num_blocks) override;
+  int num_blocks() const override { return num_blocks_; }
+  int kv_layers() const override { return mc_.num_layers; }
+  size_t k_block_bytes(int) const override { return kv_block_bytes(); }
+  size_t v_block_bytes(int) const override { return kv_block_bytes(); }
+  int64_t kv_bytes_per_block() const override { return vra_kv_per_block_bytes(&mc_, &ec_); }
+  int max_logit_rows() const override { return max_seqs_; }
   // one block of one layer's K (or V) cache: contiguous, [Hkv, BS, D] (or [Hkv, D, BS]) elements
   size_t kv_block_bytes() const { return (size_t)hkv_ * ec_.block_size * mc_.head_dim * (ec_.fp8_kvcache ? 1 : es_); }
-  void* k_cache(int l) const { return kc_[l]; }
-  void* v_cache(int l) const { return vc_[l]; }
+  void* k_cache(int l) const override { return kc_[l]; }
+  void* v_cache(int l) const override { return vc_[l]; }
   // activations are sized for max_tokens rows
-  bool init_buffers(int max_tokens, int max_seqs);
-  void set_comm(void* comm) { comm_ = comm; }
-  bool has_comm() const { return comm_ != nullptr; }
-  int world() const { return world_; }
+  bool init_buffers(int max_tokens, int max_seqs) override;
+  void set_comm(void* comm) override { comm_ = comm; }
+  bool has_comm() const override { return comm_ != nullptr; }
+  int world() const override { return world_; }
   // forward → logits (device, f32 [n_seqs, vocab]) ; returns false on argument error
   // tokens != null: the greedy token of every logits row is written there as well (out of the lm_head launch itself where the
   // kernel offers it, else by an argmax launch)
-  bool forward(const InputMetadata& md, int64_t stream, uint32_t* tokens = nullptr);
-  float* logits() const { return logits_; }
+  bool forward(const InputMetadata& md, int64_t stream, uint32_t* tokens = nullptr) override;
+  float* logits() const override { return logits_; }
   const vra_model_config& config() const { return mc_; }
   int local_heads() const { return hq_; }
   int local_kv_heads() const { return hkv_; }
-  size_t weight_bytes() const { return weight_bytes_; }
+  size_t weight_bytes() const override { return weight_bytes_; }
   // microbenchmark hooks (bench.py roofline leg): launch one decode-shaped GEMM of layer `layer`
   // which: 0 qkv(fused norm) 1 o_proj 2 gate_up 3 down 4 lm_head ; M rows
-  bool launch_gemm(int which, int layer, int M, int64_t stream);
+  bool launch_gemm(int which, int layer, int M, int64_t stream) override;
   bool lm_head(const void* xin, int rows, uint32_t* tokens, int64_t stream);
-  int64_t gemm_algorithmic_bytes(int which, int M) const;
+  int64_t gemm_algorithmic_bytes(int which, int M) const override;
   // which fused-norm launches of a step of M rows apply the RMSNorm factor in their EPILOGUE (kernel E at 1..4 rows, gemv_q4s.cuh;
   // the oracle restates that order): bit 0 = norm + q/k/v, bit 1 = norm + gate/up.  0 for every other step.
   // (steps of 5..32 rows, round 5: the launches that take ready-made operands from their producer — gate/up behind a kernel-W
   // o_proj, the q/k/v of layers >= 1 behind a kernel-W down_proj: per LAYER)
-  int norm_deferred_mask(int M, int layer = 1) const;
+  int norm_deferred_mask(int M, int layer = 1) const override;
   // Parity instrumentation of the tensor-parallel forward (tests/test_gpu_tp.py, tools/tp8_stress.py): with snapshots on, layer 0
   // of every forward leaves copies of its stages — 0 q, 1 k, 2 v (GEMM outputs, before RoPE), 3 attention output (o_proj's x),
   // 4 o_proj partial (what this rank hands to the all-reduce), 5 h after all-reduce + residual, 6 SiLU(gate)*up (down_proj's x),
   // 7 down_proj partial, 8 h after the second all-reduce — so that a deviating logit can be traced to the first stage and rank
   // that deviates from the oracle.  Off (the default): no buffers, no copies.
-  void set_tp_snapshots(int on) { snap_on_ = on != 0; snap_layer_ = on > 0 ? on - 1 : 0; }  // on = 1 + the layer to copy
-  int64_t read_tp_snapshot(int idx, void* host, int64_t max_bytes, int64_t stream);  // bytes copied, -1 on error
+  void set_tp_snapshots(int on) override { snap_on_ = on != 0; snap_layer_ = on > 0 ? on - 1 : 0; }  // on = 1 + the layer to copy
+  int64_t read_tp_snapshot(int idx, void* host, int64_t max_bytes, int64_t stream) override;  // bytes copied, -1 on error
 
  private:
   void* dalloc(size_t bytes);

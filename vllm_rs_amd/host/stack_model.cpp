@@ -1,0 +1,537 @@
+// stack_model.cpp — see stack_model.h.
+#include "stack_model.h"
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <algorithm>
+#include <sstream>
+
+#include "../csrc/stack_launch.h"
+#include "host_utils.h"
+#include "model.h"
+
+namespace vra {
+
+std::unique_ptr<ModelBase> make_model(const vra_model_config& mc, const vra_engine_config& ec, const char* spec, std::string* error) {
+  if (mc.arch == VRA_ARCH_STACK) {
+    if (!spec || !spec[0]) {
+      if (error) *error = "a layer-stack model needs its layer list (vra_engine_create_spec)";
+      return nullptr;
+    }
+    return std::unique_ptr<ModelBase>(new StackModel(mc, ec, spec));
+  }
+  return std::unique_ptr<ModelBase>(new Model(mc, ec));
+}
+
+static int round_up(int v, int m) { return (v + m - 1) / m * m; }
+
+StackModel::StackModel(const vra_model_config& mc, const vra_engine_config& ec, const char* spec) : mc_(mc), ec_(ec) {
+  dt_ = mc.dtype == VRA_F32 ? VRA_F32 : VRA_BF16;
+  es_ = dt_ == VRA_F32 ? 4 : 2;
+  if (mc.dtype != VRA_F32 && mc.dtype != VRA_BF16) spec_error_ = "layer stack: dtype must be bfloat16 or float32";
+  else if (ec.tp_world_size > 1) spec_error_ = "layer stack: tensor parallelism is not wired for this model class";
+  else if (ec.fp8_kvcache) spec_error_ = "layer stack: the cache keeps the model's element type (no fp8 cache)";
+  else parse_spec(spec);
+}
+StackModel::~StackModel() {
+  for (void* p : allocs_) (void)hipFree(p);
+}
+
+bool StackModel::parse_spec(const char* spec) {
+  std::istringstream in(spec);
+  std::string line;
+  bool have_stack = false;
+  while (std::getline(in, line)) {
+    std::istringstream ls(line);
+    std::string kind, kv;
+    if (!(ls >> kind)) continue;
+    std::map<std::string, std::string> f;
+    while (ls >> kv) {
+      const size_t eq = kv.find('=');
+      if (eq == std::string::npos) return spec_error_ = "layer stack spec: field without '=': " + kv, false;
+      f[kv.substr(0, eq)] = kv.substr(eq + 1);
+    }
+    auto num = [&](const char* k, double dflt) { return f.count(k) ? strtod(f[k].c_str(), nullptr) : dflt; };
+    if (kind == "stack") {
+      have_stack = true;
+      width_ = (int)num("width", 0), vocab_ = (int)num("vocab", 0), groups_ = (int)num("groups", 1);
+      eps_ = (float)num("eps", 1e-6), residual_mult_ = (float)num("residual_mult", 1.0), logit_scale_ = (float)num("logit_scale", 1.0);
+      pos_base_ = num("pos_base", 10000.0);
+    } else if (kind == "layer") {
+      StackLayer L;
+      L.heads = (int)num("heads", 0), L.kv_heads = (int)num("kv_heads", L.heads), L.dim = (int)num("dim", 0), L.vdim = (int)num("vdim", L.dim);
+      L.scale = (float)num("scale", L.dim > 0 ? 1.0 / sqrt((double)L.dim) : 1.0), L.softcap = (float)num("softcap", 0.0);
+      L.temp_coef = (float)num("temp_coef", 0.0), L.temp_every = (int)num("temp_every", 0), L.kv_from = (int)num("kv_from", -1);
+      const std::string mlp = f.count("mlp") ? f["mlp"] : "none";
+      L.mlp = mlp == "dense" ? 1 : (mlp == "moe" ? 2 : 0);
+      if (mlp != "dense" && mlp != "moe" && mlp != "none") return spec_error_ = "layer stack spec: unknown feed-forward kind " + mlp, false;
+      L.ff = (int)num("ff", 0), L.experts = (int)num("experts", 0), L.top = (int)num("top", 1), L.limit = (float)num("limit", 0.0);
+      L.shared_ff = (int)num("shared_ff", 0), L.shared_limit = (float)num("shared_limit", 0.0);
+      layers_.push_back(L);
+    } else {
+      return spec_error_ = "layer stack spec: unknown record " + kind, false;
+    }
+  }
+  if (!have_stack || width_ <= 0 || vocab_ <= 0 || layers_.empty()) return spec_error_ = "layer stack spec: width, vocab and at least one layer are needed", false;
+  if (groups_ < 1 || width_ % groups_) return spec_error_ = "layer stack spec: the width must split into equal norm groups", false;
+  if (width_ != mc_.hidden_size || vocab_ != mc_.vocab_size || (int)layers_.size() != mc_.num_layers)
+    return spec_error_ = "layer stack spec: width / vocab / layers differ from the model config", false;
+  for (size_t i = 0; i < layers_.size(); i++) {
+    StackLayer& L = layers_[i];
+    const std::string at = " (layer " + std::to_string(i) + ")";
+    if (L.heads <= 0 || L.kv_heads <= 0 || L.heads % L.kv_heads || L.dim <= 0 || L.vdim <= 0 || L.vdim > 256)
+      return spec_error_ = "layer stack spec: heads must be a multiple of kv_heads, sizes positive, value size at most 256" + at, false;
+    if (L.kv_from >= 0) {
+      if (L.kv_from >= (int)i) return spec_error_ = "layer stack spec: kv_from must name an earlier layer" + at, false;
+      const StackLayer& S = layers_[L.kv_from];
+      if (!S.owns_cache || S.kv_heads != L.kv_heads || S.dim != L.dim || S.vdim != L.vdim)
+        return spec_error_ = "layer stack spec: kv_from must name a layer with projections of its own and equal key / value shapes" + at, false;
+      L.cache = S.cache;
+    } else {
+      L.owns_cache = true;
+      L.cache = (int)cache_layer_.size();
+      cache_layer_.push_back((int)i);
+    }
+    if (L.mlp == 1 && L.ff <= 0) return spec_error_ = "layer stack spec: dense feed-forward without ff" + at, false;
+    if (L.mlp == 2 && (L.ff <= 0 || L.experts <= 0 || L.top < 1 || L.top > L.experts))
+      return spec_error_ = "layer stack spec: mixture of experts needs ff, experts and 1 <= top <= experts" + at, false;
+    L.ffp = round_up(L.ff, 16), L.sffp = round_up(L.shared_ff, 16);
+  }
+  return true;
+}
+
+void* StackModel::dalloc(size_t bytes) {
+  void* p = nullptr;
+  if (hipMalloc(&p, bytes ? bytes : 16) != hipSuccess) {
+    error = "hipMalloc failed for " + std::to_string(bytes) + " bytes";
+    return nullptr;
+  }
+  allocs_.push_back(p);
+  return p;
+}
+void* StackModel::upload(const void* host, size_t bytes) {
+  void* p = dalloc(bytes);
+  if (p && hipMemcpy(p, host, bytes, hipMemcpyHostToDevice) != hipSuccess) {
+    error = "hipMemcpy failed";
+    return nullptr;
+  }
+  return p;
+}
+
+// ---------------------------------------------------------------------------------------------
+// weights: tensors are staged on the host under their checkpoint names and laid out for the kernels in finalize_weights()
+// ---------------------------------------------------------------------------------------------
+bool StackModel::load_tensor(const std::string& name, const void* host, const int64_t* shape, int ndim, int elem_bytes) {
+  if (!spec_error_.empty()) return error = spec_error_, false;
+  if (finalized_) return error = "load_tensor after finalize", false;
+  if (elem_bytes != 2 && elem_bytes != 4) return error = "tensor " + name + ": 2- or 4-byte elements expected", false;
+  HostTensor t;
+  size_t n = 1;
+  for (int i = 0; i < ndim; i++) t.shape.push_back(shape[i]), n *= (size_t)shape[i];
+  t.elem_bytes = elem_bytes;
+  t.data.assign((const uint8_t*)host, (const uint8_t*)host + n * elem_bytes);
+  staged_[name] = std::move(t);
+  return true;
+}
+
+bool StackModel::need(const std::string& name, int64_t d0, int64_t d1, const HostTensor** out) {
+  auto it = staged_.find(name);
+  if (it == staged_.end()) return error = "missing tensor: " + name, false;
+  const HostTensor& t = it->second;
+  int64_t n = 1;
+  for (int64_t d : t.shape) n *= d;
+  const bool ok = d1 < 0 ? n == d0 : (t.shape.size() == 2 && t.shape[0] == d0 && t.shape[1] == d1);
+  if (!ok) return error = "tensor " + name + ": shape differs from the config", false;
+  *out = &t;
+  return true;
+}
+// small f32 tensors (norm weights, activation coefficients) whatever the checkpoint's element type
+float* StackModel::upload_f32(const HostTensor& t) {
+  const size_t n = t.data.size() / t.elem_bytes;
+  std::vector<float> f(n);
+  for (size_t i = 0; i < n; i++) {
+    if (t.elem_bytes == 4) memcpy(&f[i], t.data.data() + i * 4, 4);
+    else {
+      uint16_t b;
+      memcpy(&b, t.data.data() + i * 2, 2);
+      const uint32_t u = (uint32_t)b << 16;
+      memcpy(&f[i], &u, 4);
+    }
+  }
+  weight_bytes_ += n * 4;
+  return (float*)upload(f.data(), n * 4);
+}
+
+bool StackModel::finalize_weights() {
+  if (finalized_) return true;
+  if (!spec_error_.empty()) return error = spec_error_, false;
+  const int W = width_;
+  const size_t es = es_;
+  auto matrix = [&](const HostTensor* t) -> bool {
+    if ((size_t)t->elem_bytes != es) return error = "matrix tensors must come in the model's element type", false;
+    return true;
+  };
+  auto up_mat = [&](const std::string& name, int64_t r, int64_t c, void** dst) {
+    const HostTensor* t;
+    if (!need(name, r, c, &t) || !matrix(t)) return false;
+    weight_bytes_ += t->data.size();
+    return (*dst = upload(t->data.data(), t->data.size())) != nullptr;
+  };
+  auto up_vec = [&](const std::string& name, int64_t n, float** dst) {
+    const HostTensor* t;
+    if (!need(name, n, -1, &t)) return false;
+    return (*dst = upload_f32(*t)) != nullptr;
+  };
+  // gate / up rows of one expert -> [2 * fp][W], blocks of 16 rows alternating gate / up, zero rows beyond f
+  auto interleave = [&](const HostTensor* g, const HostTensor* u, int f, int fp, uint8_t* dst) {
+    memset(dst, 0, (size_t)2 * fp * W * es);
+    for (int r = 0; r < f; r++) {
+      const size_t blk = r / 16, i = r % 16;
+      memcpy(dst + ((2 * blk) * 16 + i) * W * es, g->data.data() + (size_t)r * W * es, W * es);
+      memcpy(dst + ((2 * blk + 1) * 16 + i) * W * es, u->data.data() + (size_t)r * W * es, W * es);
+    }
+  };
+  // down [W][f] -> [W][fp], zero columns beyond f
+  auto pad_cols = [&](const HostTensor* d, int f, int fp, uint8_t* dst) {
+    memset(dst, 0, (size_t)W * fp * es);
+    for (int r = 0; r < W; r++) memcpy(dst + (size_t)r * fp * es, d->data.data() + (size_t)r * f * es, (size_t)f * es);
+  };
+  if (!up_mat("embed", vocab_, W, &embed_) || !up_mat("head", vocab_, W, &head_) || !up_vec("final.norm", W, &final_norm_)) return false;
+  for (size_t li = 0; li < layers_.size(); li++) {
+    StackLayer& L = layers_[li];
+    const std::string p = "l" + std::to_string(li) + ".";
+    if (!up_vec(p + "norm1", W, &L.norm_w)) return false;
+    {  // q (| k | v) in one matrix: one launch projects them all
+      const HostTensor *q, *k = nullptr, *v = nullptr;
+      if (!need(p + "mix.q", L.nq(), W, &q) || !matrix(q)) return false;
+      if (L.owns_cache && (!need(p + "mix.k", L.nk(), W, &k) || !need(p + "mix.v", L.nv(), W, &v) || !matrix(k) || !matrix(v))) return false;
+      std::vector<uint8_t> cat(q->data);
+      if (k) cat.insert(cat.end(), k->data.begin(), k->data.end()), cat.insert(cat.end(), v->data.begin(), v->data.end());
+      weight_bytes_ += cat.size();
+      if (!(L.qkv = upload(cat.data(), cat.size()))) return false;
+    }
+    if (!up_mat(p + "mix.o", W, L.heads * L.vdim, &L.o)) return false;
+    if (L.mlp == 1) {
+      if (!up_mat(p + "mlp.up", L.ff, W, &L.up) || !up_mat(p + "mlp.down", W, L.ff, &L.down) || !up_vec(p + "mlp.act", 4, &L.act)) return false;
+    } else if (L.mlp == 2) {
+      const HostTensor *r, *sg = nullptr;
+      if (!need(p + "mlp.router", L.experts, W, &r) || !matrix(r)) return false;
+      if (L.shared_ff > 0 && (!need(p + "mlp.shared.sg", W, -1, &sg) || !matrix(sg))) return false;
+      std::vector<uint8_t> rt(r->data);
+      if (sg) rt.insert(rt.end(), sg->data.begin(), sg->data.end());
+      weight_bytes_ += rt.size();
+      if (!(L.router = upload(rt.data(), rt.size()))) return false;
+      std::vector<uint8_t> gu((size_t)L.experts * 2 * L.ffp * W * es), dn((size_t)L.experts * W * L.ffp * es);
+      for (int e = 0; e < L.experts; e++) {
+        const std::string pe = p + "mlp.e" + std::to_string(e) + ".";
+        const HostTensor *g, *u, *d;
+        if (!need(pe + "gate", L.ff, W, &g) || !need(pe + "up", L.ff, W, &u) || !need(pe + "down", W, L.ff, &d) || !matrix(g) || !matrix(u) || !matrix(d))
+          return false;
+        interleave(g, u, L.ff, L.ffp, gu.data() + (size_t)e * 2 * L.ffp * W * es);
+        pad_cols(d, L.ff, L.ffp, dn.data() + (size_t)e * W * L.ffp * es);
+      }
+      weight_bytes_ += gu.size() + dn.size();
+      if (!(L.e_gu = upload(gu.data(), gu.size())) || !(L.e_down = upload(dn.data(), dn.size()))) return false;
+      if (L.shared_ff > 0) {
+        const HostTensor *g, *u, *d;
+        if (!need(p + "mlp.shared.gate", L.shared_ff, W, &g) || !need(p + "mlp.shared.up", L.shared_ff, W, &u) ||
+            !need(p + "mlp.shared.down", W, L.shared_ff, &d) || !matrix(g) || !matrix(u) || !matrix(d))
+          return false;
+        std::vector<uint8_t> sgu((size_t)2 * L.sffp * W * es), sdn((size_t)W * L.sffp * es);
+        interleave(g, u, L.shared_ff, L.sffp, sgu.data());
+        pad_cols(d, L.shared_ff, L.sffp, sdn.data());
+        weight_bytes_ += sgu.size() + sdn.size();
+        if (!(L.s_gu = upload(sgu.data(), sgu.size())) || !(L.s_down = upload(sdn.data(), sdn.size()))) return false;
+      }
+    }
+  }
+  // the angle of channel pair i is p * base^(-2i / width): the factor is formed in f64 and rounded once, the product is f32
+  std::vector<float> inv((W + 1) / 2);
+  for (size_t i = 0; i < inv.size(); i++) inv[i] = (float)pow(pos_base_, -2.0 * (double)i / (double)W);
+  if (!(inv_freq_ = (float*)upload(inv.data(), inv.size() * 4))) return false;
+  staged_.clear();
+  finalized_ = hipDeviceSynchronize() == hipSuccess;
+  if (!finalized_) error = "layer stack: device error while loading weights";
+  return finalized_;
+}
+
+// random weights of the configured shapes (benchmarks, tests of the engine path): N(0, 1 / sqrt(fan in)) matrices, norm weights near 1
+bool StackModel::init_synthetic(uint64_t seed) {
+  if (!spec_error_.empty()) return error = spec_error_, false;
+  uint64_t s = seed * 0x9E3779B97F4A7C15ull + 0x1234567ull;
+  auto rnd = [&]() {  // xorshift64*; the sum of four uniforms is close enough to a normal for synthetic weights
+    s ^= s >> 12, s ^= s << 25, s ^= s >> 27;
+    return (double)((s * 0x2545F4914F6CDD1Dull) >> 11) / (double)(1ull << 53);
+  };
+  auto normal = [&]() { return (rnd() + rnd() + rnd() + rnd() - 2.0) * 1.7320508; };
+  auto put = [&](const std::string& name, int64_t r, int64_t c, double mean, double sd) {
+    const size_t n = (size_t)r * (c > 0 ? c : 1);
+    HostTensor t;
+    t.elem_bytes = (int)es_;
+    t.shape.push_back(r);
+    if (c > 0) t.shape.push_back(c);
+    t.data.resize(n * es_);
+    for (size_t i = 0; i < n; i++) {
+      const float v = (float)(mean + sd * normal());
+      if (es_ == 4) memcpy(t.data.data() + i * 4, &v, 4);
+      else {
+        const uint16_t b = host_f32_to_bf16(v);
+        memcpy(t.data.data() + i * 2, &b, 2);
+      }
+    }
+    staged_[name] = std::move(t);
+  };
+  const int W = width_;
+  put("embed", vocab_, W, 0, 1.0);
+  put("head", vocab_, W, 0, 1.0 / sqrt((double)W));
+  put("final.norm", W, 0, 1, 0.05);
+  for (size_t li = 0; li < layers_.size(); li++) {
+    const StackLayer& L = layers_[li];
+    const std::string p = "l" + std::to_string(li) + ".";
+    const double sw = 1.0 / sqrt((double)W);
+    put(p + "norm1", W, 0, 1, 0.05);
+    put(p + "mix.q", L.nq(), W, 0, sw);
+    if (L.owns_cache) put(p + "mix.k", L.nk(), W, 0, sw), put(p + "mix.v", L.nv(), W, 0, sw);
+    put(p + "mix.o", W, L.heads * L.vdim, 0, 1.0 / sqrt((double)L.heads * L.vdim));
+    if (L.mlp == 1) {
+      put(p + "mlp.up", L.ff, W, 0, sw), put(p + "mlp.down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
+      HostTensor a;
+      a.elem_bytes = 4, a.shape = {4};
+      const float c[4] = {0.6f, 0.3f, 0.1f, 0.02f};
+      a.data.assign((const uint8_t*)c, (const uint8_t*)c + 16);
+      staged_[p + "mlp.act"] = a;
+    } else if (L.mlp == 2) {
+      put(p + "mlp.router", L.experts, W, 0, sw);
+      for (int e = 0; e < L.experts; e++) {
+        const std::string pe = p + "mlp.e" + std::to_string(e) + ".";
+        put(pe + "gate", L.ff, W, 0, sw), put(pe + "up", L.ff, W, 0, sw), put(pe + "down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
+      }
+      if (L.shared_ff > 0) {
+        put(p + "mlp.shared.gate", L.shared_ff, W, 0, sw), put(p + "mlp.shared.up", L.shared_ff, W, 0, sw);
+        put(p + "mlp.shared.down", W, L.shared_ff, 0, 1.0 / sqrt((double)L.shared_ff)), put(p + "mlp.shared.sg", 1, W, 0, sw);
+      }
+    }
+  }
+  return finalize_weights();
+}
+
+// ---------------------------------------------------------------------------------------------
+// cache and buffers
+// ---------------------------------------------------------------------------------------------
+size_t StackModel::k_block_bytes(int c) const {
+  const StackLayer& L = layers_[cache_layer_[c]];
+  return (size_t)ec_.block_size * L.nk() * es_;
+}
+size_t StackModel::v_block_bytes(int c) const {
+  const StackLayer& L = layers_[cache_layer_[c]];
+  return (size_t)ec_.block_size * L.nv() * es_;
+}
+int64_t StackModel::kv_bytes_per_block() const {
+  int64_t b = 0;
+  for (size_t c = 0; c < cache_layer_.size(); c++) b += (int64_t)k_block_bytes((int)c) + (int64_t)v_block_bytes((int)c);
+  return b;
+}
+bool StackModel::init_kv_cache(int num_blocks) {
+  if (!spec_error_.empty()) return error = spec_error_, false;
+  num_blocks_ = num_blocks;
+  kc_.assign(cache_layer_.size(), nullptr);
+  vc_.assign(cache_layer_.size(), nullptr);
+  for (size_t c = 0; c < cache_layer_.size(); c++) {
+    const size_t kb = (size_t)num_blocks * k_block_bytes((int)c), vb = (size_t)num_blocks * v_block_bytes((int)c);
+    if (!(kc_[c] = dalloc(kb)) || !(vc_[c] = dalloc(vb))) return false;
+    if (hipMemset(kc_[c], 0, kb) != hipSuccess || hipMemset(vc_[c], 0, vb) != hipSuccess) return error = "kv cache clear failed", false;
+  }
+  return hipDeviceSynchronize() == hipSuccess;
+}
+
+bool StackModel::init_buffers(int max_tokens, int max_seqs) {
+  if (!spec_error_.empty()) return error = spec_error_, false;
+  max_tokens_ = max_tokens, max_seqs_ = max_seqs;
+  const size_t T = max_tokens, W = width_;
+  size_t nqkv = 0, nattn = 0, zc = 0, actc = 0, top = 0, experts = 0;
+  for (const StackLayer& L : layers_) {
+    nqkv = std::max(nqkv, (size_t)L.nqkv()), nattn = std::max(nattn, (size_t)L.heads * L.vdim);
+    if (L.mlp == 2) top = std::max(top, (size_t)L.top), experts = std::max(experts, (size_t)L.experts);
+  }
+  max_rows_ = (int)round_up((int)(T * std::max<size_t>(top, 1) + experts * 63), 64);
+  for (const StackLayer& L : layers_) {
+    if (L.mlp == 1) zc = std::max(zc, T * L.ff), actc = std::max(actc, T * L.ff);
+    if (L.mlp == 2) {
+      zc = std::max(zc, std::max((size_t)max_rows_ * 2 * L.ffp, T * 2 * L.sffp));
+      actc = std::max(actc, std::max((size_t)max_rows_ * L.ffp, T * L.sffp));
+    }
+  }
+  // logits rows: at least one per sequence; replayed traces ask for many rows of one step, so take what 256 MiB hold
+  logit_rows_cap_ = (int)std::max<size_t>(max_seqs, std::min<size_t>(T, ((size_t)256 << 20) / ((size_t)vocab_ * 4)));
+  const size_t R = logit_rows_cap_;
+  if (!(x_ = (float*)dalloc(T * W * 4)) || !(o_ = (float*)dalloc(T * W * 4)) || !(h_ = dalloc(T * W * es_)) || !(qkv_ = dalloc(T * nqkv * es_)) ||
+      !(attn_ = dalloc(T * nattn * es_)) || !(z_ = (float*)dalloc(std::max<size_t>(zc, 4) * 4)) || !(act_ = dalloc(std::max<size_t>(actc, 4) * es_)) ||
+      !(pair_out_ = (float*)dalloc(T * std::max<size_t>(top, 1) * W * 4)) || !(sh_ = (float*)dalloc(T * W * 4)) || !(xl_ = (float*)dalloc(R * W * 4)) ||
+      !(hl_ = dalloc(R * W * es_)) || !(logits_ = (float*)dalloc(R * (size_t)vocab_ * 4)))
+    return false;
+  const size_t P = T * std::max<size_t>(top, 1);
+  if (!(pair_expert_ = (int*)dalloc(P * 4)) || !(pair_weight_ = (float*)dalloc(P * 4)) || !(gate_ = (float*)dalloc(T * 4)) ||
+      !(row_token_ = (int*)dalloc((size_t)max_rows_ * 4)) || !(row_pair_ = (int*)dalloc((size_t)max_rows_ * 4)) ||
+      !(row_scale_ = (float*)dalloc((size_t)max_rows_ * 4)) || !(tile_group_ = (int*)dalloc((size_t)max_rows_ / 16 * 4)))
+    return false;
+  return hipDeviceSynchronize() == hipSuccess;
+}
+
+// ---------------------------------------------------------------------------------------------
+// forward
+// ---------------------------------------------------------------------------------------------
+static bool take_stack_err(std::string& error, const char* where) {
+  const char* e = vra_last_error();
+  if (e && e[0]) {
+    error = std::string(where) + ": " + e;
+    vra_clear_error();
+    return true;
+  }
+  return false;
+}
+
+// gate / up -> clamped gated activation -> down for `rows` logical rows (one expert per granule, or one weight set for all):
+// bf16: the activation is the epilogue of the gate / up launch; f32: product, activation and product as three launches
+bool StackModel::expert_pair(const void* a, int lda, const void* w_gu, int64_t gu_stride, const void* w_down, int64_t down_stride, int rows, int fp,
+                             int f, float limit, const int* tile_group, int granule, const int* a_row, const float* a_scale, const int* out_row,
+                             float* out, int64_t stream) {
+  const int W = width_;
+  StkGemmArgs g;
+  g.a = a, g.lda = lda, g.w = w_gu, g.w_group_stride = gu_stride, g.M = rows, g.N = 2 * fp, g.K = W;
+  g.tile_group = tile_group, g.granule = granule, g.a_row = a_row, g.a_scale = a_scale;
+  g.limit = limit;
+  const bool fused = dt_ == VRA_BF16 && W % 8 == 0 && lda % 8 == 0;
+  if (fused) {
+    g.epi = 1, g.out = act_, g.ldo = fp;
+    vra_stack_gemm(g, dt_, stream);
+  } else {
+    g.out = z_, g.ldo = 2 * fp, g.out_f32 = 1;
+    vra_stack_gemm(g, dt_, stream);
+    vra_stack_gated_act(z_, act_, rows, f, limit, 1.702f, dt_, stream);
+  }
+  StkGemmArgs d;
+  d.a = act_, d.lda = fp, d.w = w_down, d.w_group_stride = down_stride, d.M = rows, d.N = W, d.K = fp;
+  d.out = out, d.ldo = W, d.out_f32 = 1;
+  d.tile_group = tile_group, d.granule = granule, d.out_row = out_row;
+  // rows of a granule that hold no pair are neither read nor written: a_row of the first launch marks them, the second sees them through out_row
+  vra_stack_gemm(d, dt_, stream);
+  return !take_stack_err(error, "expert feed-forward");
+}
+
+bool StackModel::feed_forward(const StackLayer& L, int T, int64_t stream) {
+  const int W = width_;
+  if (L.mlp == 1) {
+    StkGemmArgs u;
+    u.a = h_, u.lda = W, u.w = L.up, u.M = T, u.N = L.ff, u.K = W, u.out = z_, u.ldo = L.ff, u.out_f32 = 1;
+    vra_stack_gemm(u, dt_, stream);
+    vra_stack_polynorm(z_, act_, L.act, T, L.ff, eps_, dt_, stream);
+    StkGemmArgs d;
+    d.a = act_, d.lda = L.ff, d.w = L.down, d.M = T, d.N = W, d.K = L.ff, d.out = pair_out_, d.ldo = W, d.out_f32 = 1;
+    vra_stack_gemm(d, dt_, stream);
+    vra_stack_residual_combine(x_, o_, pair_out_, 1, nullptr, nullptr, residual_mult_, T, W, stream);
+    return !take_stack_err(error, "dense feed-forward");
+  }
+  if (L.mlp == 2) {
+    const int P = T * L.top;
+    const int granule = vra_stack_gemm_granule(P, L.experts);
+    const int rows = round_up(P + L.experts * (granule - 1), granule);
+    if (rows > max_rows_) return error = "feed-forward: more expert rows than the buffers hold", false;
+    vra_stack_moe_sort(pair_expert_, pair_weight_, P, L.top, L.experts, granule, rows, row_token_, row_scale_, row_pair_, tile_group_, stream);
+    if (take_stack_err(error, "expert rows")) return false;
+    if (!expert_pair(h_, W, L.e_gu, (int64_t)2 * L.ffp * W, L.e_down, (int64_t)W * L.ffp, rows, L.ffp, L.ff, L.limit, tile_group_, granule, row_token_,
+                     row_scale_, row_pair_, pair_out_, stream))
+      return false;
+    if (L.shared_ff > 0 &&
+        !expert_pair(h_, W, L.s_gu, 0, L.s_down, 0, T, L.sffp, L.shared_ff, L.shared_limit, nullptr, 0, nullptr, nullptr, nullptr, sh_, stream))
+      return false;
+    vra_stack_residual_combine(x_, o_, pair_out_, L.top, L.shared_ff > 0 ? sh_ : nullptr, L.shared_ff > 0 ? gate_ : nullptr, residual_mult_, T, W, stream);
+    return !take_stack_err(error, "mixture of experts");
+  }
+  vra_stack_residual_combine(x_, o_, nullptr, 0, nullptr, nullptr, residual_mult_, T, W, stream);
+  return !take_stack_err(error, "residual");
+}
+
+bool StackModel::forward(const InputMetadata& md, int64_t stream, uint32_t* tokens) {
+  if (!finalized_) return error = "forward before the weights are complete", false;
+  const int T = md.n_tokens, B = md.n_seqs, W = width_;
+  if (T <= 0 || T > max_tokens_ || B <= 0 || B > max_seqs_) return error = "forward: batch out of range", false;
+  if (!md.is_prefill && T != B) return error = "forward: a decode step carries one token per sequence", false;
+  error.clear();
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (trace_on_) {
+    const size_t need_b = layers_.size() * (size_t)T * W * 4;
+    if (trace_cap_ < need_b) {
+      if (!(trace_ = (float*)dalloc(need_b))) return false;
+      trace_cap_ = need_b;
+    }
+    trace_bytes_ = need_b;
+  }
+  vra_stack_embed_sinpos(md.input_ids, md.positions, embed_, inv_freq_, x_, T, W, vocab_, dt_, stream);
+  if (take_stack_err(error, "embedding")) return false;
+  for (size_t li = 0; li < layers_.size(); li++) {
+    const StackLayer& L = layers_[li];
+    // h = norm(x); a mixture-of-experts layer's router (and its shared expert's gate) reads h inside the same launch
+    StkNormArgs n;
+    n.x = x_, n.w = L.norm_w, n.h = h_, n.T = T, n.W = W, n.groups = groups_, n.eps = eps_;
+    if (L.mlp == 2) {
+      n.router_w = L.router, n.n_router = L.experts, n.top = L.top, n.gate_row = L.shared_ff > 0;
+      n.pair_expert = pair_expert_, n.pair_weight = pair_weight_, n.gate_out = gate_;
+    }
+    vra_stack_group_norm(n, dt_, stream);
+    // q (| k | v) in one launch
+    const int nqkv = L.nqkv();
+    StkGemmArgs p;
+    p.a = h_, p.lda = W, p.w = L.qkv, p.M = T, p.N = nqkv, p.K = W, p.out = qkv_, p.ldo = nqkv;
+    vra_stack_gemm(p, dt_, stream);
+    if (L.owns_cache)
+      vra_stack_kv_store((const char*)qkv_ + (size_t)L.nq() * es_, (const char*)qkv_ + (size_t)(L.nq() + L.nk()) * es_, nqkv, kc_[L.cache], vc_[L.cache],
+                         md.slot_mapping, T, L.nk(), L.nv(), dt_, stream);
+    StkAttnArgs a;
+    a.q = qkv_, a.ldq = nqkv, a.out = attn_, a.kc = kc_[L.cache], a.vc = vc_[L.cache];
+    a.positions = md.positions, a.block_tables = md.block_tables, a.context_lens = md.context_lens;
+    a.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
+    a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = L.heads, a.G = L.kv_heads, a.dim = L.dim, a.vdim = L.vdim;
+    a.BS = ec_.block_size, a.max_blocks = md.max_blocks;
+    a.scale = L.scale, a.softcap = L.softcap, a.temp_coef = L.temp_coef, a.temp_every = L.temp_every;
+    vra_stack_attention(a, dt_, stream);
+    StkGemmArgs o;
+    o.a = attn_, o.lda = L.heads * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = L.heads * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;
+    vra_stack_gemm(o, dt_, stream);
+    if (take_stack_err(error, "mixer")) return false;
+    if (!feed_forward(L, T, stream)) return false;
+    if (trace_on_ && hipMemcpyAsync(trace_ + li * (size_t)T * W, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st) != hipSuccess)
+      return error = "layer trace copy failed", false;
+  }
+  // the rows whose logits are wanted -> final norm -> head
+  const float* xin = x_;
+  int rows = T;
+  const uint32_t* sel = md.n_logit_rows > 0 ? md.logit_rows : (md.is_prefill ? md.last_token_rows : nullptr);
+  if (sel) {
+    rows = md.n_logit_rows > 0 ? md.n_logit_rows : B;
+    if (rows > logit_rows_cap_) return error = "forward: more logit rows than the logits buffer holds", false;
+    vra_stack_gather_rows_f32(x_, sel, xl_, rows, W, stream);
+    xin = xl_;
+  } else if (rows > logit_rows_cap_) {
+    return error = "forward: more logit rows than the logits buffer holds", false;
+  }
+  StkNormArgs fn;
+  fn.x = xin, fn.w = final_norm_, fn.h = hl_, fn.T = rows, fn.W = W, fn.groups = groups_, fn.eps = eps_;
+  vra_stack_group_norm(fn, dt_, stream);
+  StkGemmArgs hd;
+  hd.a = hl_, hd.lda = W, hd.w = head_, hd.M = rows, hd.N = vocab_, hd.K = W, hd.out = logits_, hd.ldo = vocab_, hd.out_f32 = 1, hd.alpha = logit_scale_;
+  vra_stack_gemm(hd, dt_, stream);
+  if (tokens) vra_argmax_f32(logits_, tokens, rows, vocab_, stream);
+  return !take_stack_err(error, "head");
+}
+
+int64_t StackModel::read_layer_trace(void* host, int64_t max_bytes, int64_t stream) {
+  if (!trace_ || !host || (int64_t)trace_bytes_ > max_bytes) return -1;
+  hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+  if (hipMemcpyAsync(host, trace_, trace_bytes_, hipMemcpyDeviceToHost, st) != hipSuccess || hipStreamSynchronize(st) != hipSuccess) return -1;
+  return (int64_t)trace_bytes_;
+}
+
+}  // namespace vra

@@ -627,6 +627,30 @@ int32_t vra_engine_replay_step(void* eng, int32_t n_entries, const int64_t* h_re
 void vra_engine_debug_layer_trace(void* eng, int32_t on);
 int64_t vra_engine_debug_read_layer_trace(void* eng, void* h_out, int64_t max_bytes);
 
+/* The operators of layer-stack models one by one (vllm_rs_amd/csrc/stack_launch.h states each; dtype VRA_BF16 or VRA_F32; device
+ * pointers, asynchronous on `stream`, errors through vra_last_error). */
+void vra_stack_op_embed_sinpos(const uint32_t* ids, const int64_t* positions, const void* embed, const float* inv_freq, float* x,
+                               int32_t T, int32_t W, int32_t V, int32_t dtype, int64_t stream);
+void vra_stack_op_group_norm(const float* x, const float* w, void* h, int32_t T, int32_t W, int32_t groups, float eps,
+                             const void* router_w, int32_t n_router, int32_t top, int32_t gate_row, int32_t* pair_expert,
+                             float* pair_weight, float* gate_out, int32_t dtype, int64_t stream);
+void vra_stack_op_gemm(const void* a, int32_t lda, const void* w, int64_t w_group_stride, void* out, int32_t ldo, int32_t out_f32,
+                       int32_t M, int32_t N, int32_t K, float alpha, const int32_t* tile_group, int32_t granule, const int32_t* a_row,
+                       const float* a_scale, const int32_t* out_row, int32_t epi, float limit, int32_t dtype, int64_t stream);
+void vra_stack_op_moe_sort(const int32_t* pair_expert, const float* pair_weight, int32_t P, int32_t top, int32_t n_groups,
+                           int32_t granule, int32_t max_rows, int32_t* row_token, float* row_scale, int32_t* row_pair,
+                           int32_t* tile_group, int64_t stream);
+void vra_stack_op_gated_act(const float* gu, void* out, int32_t M, int32_t F, float limit, float act_alpha, int32_t dtype, int64_t stream);
+void vra_stack_op_polynorm(const float* z, void* out, const float* coef, int32_t M, int32_t F, float eps, int32_t dtype, int64_t stream);
+void vra_stack_op_residual_combine(float* x, const float* o, const float* p1, int32_t n1, const float* p2, const float* gate,
+                                   float mult, int32_t T, int32_t W, int64_t stream);
+void vra_stack_op_kv_store(const void* k, const void* v, int32_t ld, void* kc, void* vc, const int64_t* slots, int32_t T,
+                           int32_t kdim, int32_t vdim, int32_t dtype, int64_t stream);
+void vra_stack_op_attention(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                            const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                            int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks,
+                            float scale, float softcap, float temp_coef, int32_t temp_every, int32_t dtype, int64_t stream);
+
 /* decode-step microbenchmark hook used by bench.py: runs `steps` decode steps of the current
  * running batch back to back (graph replay when enabled) and returns elapsed ms measured with HIP
  * events on the engine stream; tokens are sampled and appended exactly as in vra_engine_step. */

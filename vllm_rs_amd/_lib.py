@@ -197,6 +197,16 @@ def load():
     _sig(lib, "vra_pc_evict_blocks", c_i32, P, c_i32, P, c_i32)
     _sig(lib, "vra_engine_create", P, MC, EC)
     _sig(lib, "vra_engine_destroy", None, P)
+    _sig(lib, "vra_stack_op_embed_sinpos", None, P, P, P, P, P, c_i32, c_i32, c_i32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_group_norm", None, P, P, P, c_i32, c_i32, c_i32, c_f32, P, c_i32, c_i32, c_i32, P, P, P, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_gemm", None, P, c_i32, P, c_i64, P, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, P, c_i32, P, P, P, c_i32, c_f32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_moe_sort", None, P, P, c_i32, c_i32, c_i32, c_i32, c_i32, P, P, P, P, c_i64)
+    _sig(lib, "vra_stack_op_gated_act", None, P, P, c_i32, c_i32, c_f32, c_f32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_polynorm", None, P, P, P, c_i32, c_i32, c_f32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_residual_combine", None, P, P, P, c_i32, P, P, c_f32, c_i32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_kv_store", None, P, P, c_i32, P, P, P, c_i32, c_i32, c_i32, c_i32, c_i64)
+    _sig(lib, "vra_stack_op_attention", None, P, c_i32, P, P, P, P, P, P, P, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
+         c_f32, c_f32, c_f32, c_i32, c_i32, c_i64)
     _sig(lib, "vra_engine_create_spec", P, MC, EC, C.c_char_p)
     _sig(lib, "vra_engine_replay_step", c_i32, P, c_i32, P, P, P, P, P, c_i32, P, P)
     _sig(lib, "vra_engine_debug_layer_trace", None, P, c_i32)

@@ -701,3 +701,54 @@ void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream) {
   }
 #undef STK_PF
 }
+
+// ================================================================================================ C entry points (one operator each)
+extern "C" void vra_stack_op_embed_sinpos(const uint32_t* ids, const int64_t* positions, const void* embed, const float* inv_freq, float* x, int32_t T,
+                                          int32_t W, int32_t V, int32_t dtype, int64_t stream) {
+  vra_stack_embed_sinpos(ids, positions, embed, inv_freq, x, T, W, V, dtype, stream);
+}
+extern "C" void vra_stack_op_group_norm(const float* x, const float* w, void* h, int32_t T, int32_t W, int32_t groups, float eps, const void* router_w,
+                                        int32_t n_router, int32_t top, int32_t gate_row, int32_t* pair_expert, float* pair_weight, float* gate_out,
+                                        int32_t dtype, int64_t stream) {
+  StkNormArgs a;
+  a.x = x, a.w = w, a.h = h, a.T = T, a.W = W, a.groups = groups, a.eps = eps;
+  a.router_w = router_w, a.n_router = n_router, a.top = top, a.gate_row = gate_row;
+  a.pair_expert = pair_expert, a.pair_weight = pair_weight, a.gate_out = gate_out;
+  vra_stack_group_norm(a, dtype, stream);
+}
+extern "C" void vra_stack_op_gemm(const void* a, int32_t lda, const void* w, int64_t w_group_stride, void* out, int32_t ldo, int32_t out_f32, int32_t M,
+                                  int32_t N, int32_t K, float alpha, const int32_t* tile_group, int32_t granule, const int32_t* a_row,
+                                  const float* a_scale, const int32_t* out_row, int32_t epi, float limit, int32_t dtype, int64_t stream) {
+  StkGemmArgs g;
+  g.a = a, g.lda = lda, g.w = w, g.w_group_stride = w_group_stride, g.out = out, g.ldo = ldo, g.out_f32 = out_f32, g.M = M, g.N = N, g.K = K;
+  g.alpha = alpha, g.tile_group = tile_group, g.granule = granule, g.a_row = a_row, g.a_scale = a_scale, g.out_row = out_row, g.epi = epi, g.limit = limit;
+  vra_stack_gemm(g, dtype, stream);
+}
+extern "C" void vra_stack_op_moe_sort(const int32_t* pair_expert, const float* pair_weight, int32_t P, int32_t top, int32_t n_groups, int32_t granule,
+                                      int32_t max_rows, int32_t* row_token, float* row_scale, int32_t* row_pair, int32_t* tile_group, int64_t stream) {
+  vra_stack_moe_sort(pair_expert, pair_weight, P, top, n_groups, granule, max_rows, row_token, row_scale, row_pair, tile_group, stream);
+}
+extern "C" void vra_stack_op_gated_act(const float* gu, void* out, int32_t M, int32_t F, float limit, float act_alpha, int32_t dtype, int64_t stream) {
+  vra_stack_gated_act(gu, out, M, F, limit, act_alpha, dtype, stream);
+}
+extern "C" void vra_stack_op_polynorm(const float* z, void* out, const float* coef, int32_t M, int32_t F, float eps, int32_t dtype, int64_t stream) {
+  vra_stack_polynorm(z, out, coef, M, F, eps, dtype, stream);
+}
+extern "C" void vra_stack_op_residual_combine(float* x, const float* o, const float* p1, int32_t n1, const float* p2, const float* gate, float mult,
+                                              int32_t T, int32_t W, int64_t stream) {
+  vra_stack_residual_combine(x, o, p1, n1, p2, gate, mult, T, W, stream);
+}
+extern "C" void vra_stack_op_kv_store(const void* k, const void* v, int32_t ld, void* kc, void* vc, const int64_t* slots, int32_t T, int32_t kdim,
+                                      int32_t vdim, int32_t dtype, int64_t stream) {
+  vra_stack_kv_store(k, v, ld, kc, vc, slots, T, kdim, vdim, dtype, stream);
+}
+extern "C" void vra_stack_op_attention(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                       const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                                       int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks, float scale,
+                                       float softcap, float temp_coef, int32_t temp_every, int32_t dtype, int64_t stream) {
+  StkAttnArgs a;
+  a.q = q, a.ldq = ldq, a.out = out, a.kc = kc, a.vc = vc, a.positions = positions, a.block_tables = block_tables, a.context_lens = context_lens;
+  a.cu_q = cu_q, a.B = B, a.T = T, a.max_q = max_q, a.H = H, a.G = G, a.dim = dim, a.vdim = vdim, a.BS = BS, a.max_blocks = max_blocks;
+  a.scale = scale, a.softcap = softcap, a.temp_coef = temp_coef, a.temp_every = temp_every;
+  vra_stack_attention(a, dtype, stream);
+}

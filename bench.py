@@ -47,6 +47,8 @@ def parse():
     ap.add_argument("--no-graph", action="store_true", help="eager launches (rocprofv3 kernel tracing crashes on hipGraph replay)")
     ap.add_argument("--blocks", type=int, default=8192, help="KV blocks (64 tokens each); 0 = kv_fraction of free HBM")
     ap.add_argument("--tp", type=int, default=0, help="run ONE tensor-parallel engine over this many ranks (spawns its own runner processes)")
+    ap.add_argument("--design", default="", help="'ditilix': prefill / decode throughput of the layer-stack model class beside the dense "
+                    "Llama of the same widths (vllm_rs_amd/stack_bench.py) instead of the default workload")
     return ap.parse_args()
 
 
@@ -724,6 +726,13 @@ def tp_main(a):
 
 def main():
     a = parse()
+    if a.design:
+        if a.design.lower() != "ditilix":
+            raise SystemExit(f"bench.py: unknown --design {a.design!r} (ditilix)")
+        from vllm_rs_amd import stack_bench
+        stack_bench.main(steps=min(a.steps, 64), warmup=min(a.warmup, 8), graph=not a.no_graph,
+                         sizes=[a.model] if a.model in stack_bench.SIZES else None)  # --model <size name>: that size alone
+        return 0
     if a.tp > 1:
         return tp_main(a)
     if "WORLD_SIZE" not in os.environ and a.gpus > 1:

@@ -308,6 +308,83 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
   }
 }
 
+// Steps of up to 32 rows (decoding): the weights are the whole traffic, so a workgroup takes only 32 output columns and its 8 waves
+// take an eighth of K each (whole K-steps of 32, ascending inside a wave); the 8 partial tiles meet in LDS and are summed in wave order.
+// One fixed order for a given K — another one than the large-M kernel's single chain, so the two agree to rounding, not to the bit.
+template <bool SCALED>
+__global__ __launch_bounds__(512) void stk_gemm_mfma_small_kernel(StkGemmArgs g) {
+  __shared__ float part[8][16 * 32];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, rq = lane & 15, oct = lane >> 4;
+  int group = 0;
+  if (g.tile_group) {
+    group = g.tile_group[blockIdx.x];
+    if (group < 0) return;
+  }
+  const uint16_t* A = (const uint16_t*)g.a;
+  const uint16_t* Wt = (const uint16_t*)g.w + (int64_t)group * g.w_group_stride;
+  const int m_base = blockIdx.x * 16, n_base = blockIdx.y * 32;
+  const int r = m_base + rq;
+  const int idx = r < g.M ? (g.a_row ? g.a_row[r] : r) : -1;
+  const uint16_t* ap = A + (int64_t)(idx >= 0 ? idx : 0) * g.lda;
+  const float asc = SCALED && idx >= 0 ? g.a_scale[r] : 1.f;
+  const uint16_t* wp[2];
+  bool wv[2];
+  for (int nt = 0; nt < 2; nt++) {
+    const int n = n_base + nt * 16 + rq;
+    wv[nt] = n < g.N;
+    wp[nt] = Wt + (int64_t)(n < g.N ? n : 0) * g.K;
+  }
+  const int ksteps = (g.K + 31) / 32, per = (ksteps + 7) / 8;
+  const int k_lo = wave * per * 32, k_hi = min(g.K, (wave + 1) * per * 32);
+  f32x4 acc[2] = {vra_zero_acc(), vra_zero_acc()};
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
+    const int k = k0 + oct * 8;
+    const bool kin = k < g.K;
+    const int kc = kin ? k : 0;
+    u32x4 af = *(const u32x4*)(ap + kc);
+    if (SCALED) {
+      for (int i = 0; i < 4; i++) af[i] = BF16::pack2(__uint_as_float(af[i] << 16) * asc, __uint_as_float(af[i] & 0xffff0000u) * asc);
+    }
+    af = (idx >= 0 && kin) ? af : zero4;
+    for (int nt = 0; nt < 2; nt++) {
+      const u32x4 v = *(const u32x4*)(wp[nt] + kc);
+      const u32x4 wf = (wv[nt] && kin) ? v : zero4;
+      BF16::mfma(acc[nt], __builtin_bit_cast(s16x8, wf), __builtin_bit_cast(s16x8, af));
+    }
+  }
+  VRA_MFMA_DRAIN();
+  for (int nt = 0; nt < 2; nt++)
+    for (int j = 0; j < 4; j++) part[wave][rq * 32 + nt * 16 + oct * 4 + j] = acc[nt][j];
+  __syncthreads();
+  const int e = threadIdx.x, m = e >> 5, c = e & 31;  // one output element per thread
+  const int row = m_base + m;
+  if (row >= g.M) return;
+  const int ridx = g.a_row ? g.a_row[row] : row;
+  if (ridx < 0) return;
+  const int orow = g.out_row ? g.out_row[row] : row;
+  if (orow < 0) return;
+  auto total = [&](int col) {
+    float s = part[0][m * 32 + col];
+    for (int w = 1; w < 8; w++) s += part[w][m * 32 + col];
+    return s;
+  };
+  if (g.epi == 1) {
+    if (c >= 16) return;
+    const int n = n_base / 2 + c;
+    if (n >= g.N / 2) return;
+    const float y = gated_pair(total(c), total(16 + c), g.limit, g.act_alpha);
+    if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = y;
+    else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(y);
+  } else {
+    const int n = n_base + c;
+    if (n >= g.N) return;
+    const float v = total(c) * g.alpha;
+    if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = v;
+    else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(v);
+  }
+}
+
 // ------------------------------------------------------------------------------------------------ activations
 template <typename T>
 __global__ __launch_bounds__(256) void stk_gated_act_kernel(const float* gu, T* out, int F, float limit, float act_alpha) {
@@ -487,38 +564,195 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
   }
 }
 
-// One decoded token per sequence: a workgroup per (sequence, query head); its 4 waves take the 64-key tiles of the context in turn,
-// read K rows straight from the cache (lane = key) and V rows channel-wise (lane = channel), and meet once in LDS.
+// bf16 models, key size a multiple of 8 and value size a multiple of 16: the same operator on the matrix cores.
+// A workgroup of 4 waves owns 64 query rows of one head (16 per wave) and walks the keys in tiles of 32 from key 0.
+//   S^T = K . Q^T   A operand = K rows straight from the cache (lane = (key rq, channel octet oct)), B = Q fragments kept in registers;
+//                   the lane ends up with query row rq and keys oct * 4 + j of both 16-key halves: 8 scores, all in f32 — temperature,
+//                   scale, soft cap, mask, running maximum (two xor shuffles join the 4 lanes of a row) and exponentials;
+//   O^T += V^T . P^T  A operand = the V tile, transposed once per workgroup into LDS with the keys in the order the lanes hold their
+//                   scores (position = oct * 8 + half * 4 + j), B = the lane's own 8 weights.  The weights stay f32 in effect: each is
+//                   split into a bf16 head and a bf16 tail (p = hi + lo to 2^-17) and the product runs twice.
+// Every sum goes tile by tile from key 0 with a fixed lane pattern: the result of a row does not depend on the portion it came in.
+template <int DC, int VT>
+__global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs a) {
+  constexpr int KT = 32, VLD = KT + 8;  // LDS row of a value channel: 32 positions + 8 (rows stay 16-byte aligned, lanes spread over banks)
+  __shared__ __attribute__((aligned(16))) uint16_t vt[VT * 16 * VLD];
+  const int dim = a.dim, vdim = a.vdim;
+  const int b = blockIdx.y, h = blockIdx.z, g = h / (a.H / a.G);
+  const int q0 = a.cu_q[b], q1 = a.cu_q[b + 1];
+  const int t0 = q0 + blockIdx.x * 64;
+  if (t0 >= q1) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rq = lane & 15, oct = lane >> 4;
+  const int tq = t0 + wave * 16 + rq;  // this lane's query row
+  const bool qv = tq < q1;
+  const int64_t pq = qv ? a.positions[tq] : -1;
+  const uint16_t* q = (const uint16_t*)a.q;
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  u32x4 qf[DC];
+  for (int c = 0; c < DC; c++) {
+    const int ch = c * 32 + oct * 8;
+    const bool ok = qv && ch < dim;
+    const u32x4 v = *(const u32x4*)(q + (size_t)(ok ? tq : q0) * a.ldq + h * dim + (ok ? ch : 0));
+    qf[c] = ok ? v : zero4;
+  }
+  const float sc = a.scale * q_temperature(pq < 0 ? 0 : pq, a.temp_coef, a.temp_every);
+  // keys this workgroup needs: up to the largest position of its rows
+  int64_t pmax = pq;
+  for (int o = 32; o > 0; o >>= 1) pmax = max(pmax, (int64_t)__shfl_xor((long long)pmax, o, 64));
+  __shared__ long long wmax[4];
+  if (lane == 0) wmax[wave] = pmax;
+  __syncthreads();
+  const int64_t gmax = max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3]));
+  const int n_keys = (int)min((int64_t)a.context_lens[b], gmax + 1);
+  const int n_keys_wave = (int)min((int64_t)n_keys, pmax + 1);
+  const uint16_t* kc = (const uint16_t*)a.kc;
+  const uint16_t* vc = (const uint16_t*)a.vc;
+  const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
+  const int kdim = a.G * dim, vd_all = a.G * vdim;
+  f32x4 acc[VT];
+  for (int t = 0; t < VT; t++) acc[t] = vra_zero_acc();
+  float m = -INFINITY, l = 0.f;
+  for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
+    __syncthreads();
+    // V tile -> LDS, transposed: item = (key, 8 channels)
+    for (int i = tid; i < KT * (VT * 2); i += 256) {
+      const int kl = i / (VT * 2), c8 = (i % (VT * 2)) * 8, key = kt0 + kl;
+      u32x4 v = zero4;
+      if (key < n_keys && c8 < vdim) {
+        const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
+        v = *(const u32x4*)(vc + slot * vd_all + g * vdim + c8);
+      }
+      const int pos = ((kl & 15) >> 2) * 8 + (kl >> 4) * 4 + (kl & 3);
+      for (int e = 0; e < 4; e++) {
+        vt[(c8 + 2 * e) * VLD + pos] = (uint16_t)(v[e] & 0xffffu);
+        vt[(c8 + 2 * e + 1) * VLD + pos] = (uint16_t)(v[e] >> 16);
+      }
+    }
+    __syncthreads();
+    if (kt0 >= n_keys_wave) continue;  // (wave-uniform: nothing of this tile is visible to the wave's rows)
+    // scores of the two 16-key halves
+    f32x4 s[2];
+    for (int u = 0; u < 2; u++) {
+      const int key = kt0 + u * 16 + rq;
+      const bool kv = key < n_keys;
+      const int64_t slot = kv ? (int64_t)bt[key / a.BS] * a.BS + key % a.BS : 0;
+      const uint16_t* kr = kc + slot * kdim + g * dim;
+      s[u] = vra_zero_acc();
+      for (int c = 0; c < DC; c++) {
+        const int ch = c * 32 + oct * 8;
+        const bool ok = kv && ch < dim;
+        const u32x4 kf = *(const u32x4*)(kr + (ok ? ch : 0));
+        const u32x4 kz = ok ? kf : zero4;
+        BF16::mfma(s[u], __builtin_bit_cast(s16x8, kz), __builtin_bit_cast(s16x8, qf[c]));
+      }
+    }
+    VRA_MFMA_DRAIN();
+    float sv[8];
+    float tmax = -INFINITY;
+    for (int u = 0; u < 2; u++)
+      for (int j = 0; j < 4; j++) {
+        const int key = kt0 + u * 16 + oct * 4 + j;
+        float x = -INFINITY;
+        if (key <= pq && key < n_keys) x = cap_score(s[u][j] * sc, a.softcap);
+        sv[u * 4 + j] = x;
+        tmax = fmaxf(tmax, x);
+      }
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float mn = fmaxf(m, tmax);
+    float corr = 1.f, psum = 0.f, pv[8];
+    for (int i = 0; i < 8; i++) pv[i] = 0.f;
+    if (mn > -INFINITY) {
+      corr = m > -INFINITY ? expf(m - mn) : 0.f;
+      for (int i = 0; i < 8; i++) {
+        pv[i] = sv[i] > -INFINITY ? expf(sv[i] - mn) : 0.f;
+        psum += pv[i];
+      }
+    }
+    l = l * corr + psum;
+    m = mn;
+    u32x4 phi, plo;
+    for (int e = 0; e < 4; e++) {
+      const float a0 = pv[2 * e], a1 = pv[2 * e + 1];
+      const uint32_t hi = BF16::pack2(a0, a1);
+      phi[e] = hi;
+      plo[e] = BF16::pack2(a0 - __uint_as_float(hi << 16), a1 - __uint_as_float(hi & 0xffff0000u));
+    }
+    for (int t = 0; t < VT; t++) {
+      acc[t][0] *= corr, acc[t][1] *= corr, acc[t][2] *= corr, acc[t][3] *= corr;
+    }
+    for (int t = 0; t < VT; t++) {
+      const u32x4 vf = *(const u32x4*)(vt + (t * 16 + rq) * VLD + oct * 8);
+      BF16::mfma(acc[t], __builtin_bit_cast(s16x8, vf), __builtin_bit_cast(s16x8, phi));
+      BF16::mfma(acc[t], __builtin_bit_cast(s16x8, vf), __builtin_bit_cast(s16x8, plo));
+    }
+    VRA_MFMA_DRAIN();
+  }
+  l += __shfl_xor(l, 16, 64);
+  l += __shfl_xor(l, 32, 64);
+  if (!qv) return;
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  uint16_t* out = (uint16_t*)a.out + (size_t)tq * a.H * vdim + h * vdim;
+  for (int t = 0; t < VT; t++)
+    for (int j = 0; j < 4; j++) {
+      const int c = t * 16 + oct * 4 + j;
+      if (c < vdim) out[c] = BF16::from_f32(acc[t][j] * inv);
+    }
+}
+
+// One decoded token per sequence: a workgroup per (sequence, query head); its 8 waves take the 64-key tiles of the context in turn,
+// read K rows straight from the cache (lane = key, 16 bytes a load where the row allows) and V rows channel-wise (lane = channel), and
+// meet once in LDS.  The order of the sums depends on the context length alone.
+#define STK_DW 8
 template <typename T>
-__global__ __launch_bounds__(256) void stk_attn_decode_kernel(StkAttnArgs a) {
+__device__ __forceinline__ float stk_dot_row(const float* qs, const T* kr, int dim) {
+  float d0 = 0.f;
+  for (int d = 0; d < dim; d++) d0 = fmaf(qs[d], El<T>::ld(kr + d), d0);
+  return d0;
+}
+template <>
+__device__ __forceinline__ float stk_dot_row<uint16_t>(const float* qs, const uint16_t* kr, int dim) {
+  float d0 = 0.f;
+  if (dim % 8 == 0 && ((uintptr_t)kr % 16) == 0) {
+    for (int d = 0; d < dim; d += 8) {
+      const u32x4 v = *(const u32x4*)(kr + d);
+      for (int e = 0; e < 4; e++) {
+        d0 = fmaf(qs[d + 2 * e], __uint_as_float(v[e] << 16), d0);
+        d0 = fmaf(qs[d + 2 * e + 1], __uint_as_float(v[e] & 0xffff0000u), d0);
+      }
+    }
+    return d0;
+  }
+  for (int d = 0; d < dim; d++) d0 = fmaf(qs[d], BF16::to_f32(kr[d]), d0);
+  return d0;
+}
+template <typename T>
+__global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArgs a) {
   extern __shared__ float lds[];
   const int dim = a.dim, vdim = a.vdim;
-  float* qs = lds;                 // [dim]
-  float* ps = qs + dim;            // [4][64]
-  float* ms = ps + 4 * 64;         // [4] max, [4] sum
-  float* os = ms + 8;              // [4][vdim]
+  float* qs = lds;                     // [dim]
+  float* ps = qs + dim;                // [waves][64]
+  float* ms = ps + STK_DW * 64;        // [waves] max, [waves] sum
+  float* os = ms + 2 * STK_DW;         // [waves][vdim]
   const int b = blockIdx.x, h = blockIdx.y, g = h / (a.H / a.G);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t p = a.positions[b];
   const int n_keys = (int)min((int64_t)a.context_lens[b], p + 1);
   const T* q = (const T*)a.q + (size_t)b * a.ldq + h * dim;
   const float temp = q_temperature(p, a.temp_coef, a.temp_every);
-  for (int d = tid; d < dim; d += 256) qs[d] = El<T>::ld(q + d) * temp;
+  for (int d = tid; d < dim; d += 64 * STK_DW) qs[d] = El<T>::ld(q + d) * temp;
   __syncthreads();
   const T* kc = (const T*)a.kc;
   const T* vc = (const T*)a.vc;
   const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
   const int kdim = a.G * dim, vd_all = a.G * vdim;
   float m = -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
-  for (int kt0 = wave * 64; kt0 < n_keys; kt0 += 4 * 64) {
+  for (int kt0 = wave * 64; kt0 < n_keys; kt0 += STK_DW * 64) {
     const int key = kt0 + lane;
     float s = -INFINITY;
     if (key < n_keys) {
       const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
-      const T* kr = kc + slot * kdim + g * dim;
-      float d0 = 0.f;
-      for (int d = 0; d < dim; d++) d0 = fmaf(qs[d], El<T>::ld(kr + d), d0);
-      s = cap_score(d0 * a.scale, a.softcap);
+      s = cap_score(stk_dot_row<T>(qs, kc + slot * kdim + g * dim, dim) * a.scale, a.softcap);
     }
     const float mn = fmaxf(m, wave_max(s));  // (the tile's first key exists: mn is finite)
     const float pj = s > -INFINITY ? expf(s - mn) : 0.f;
@@ -530,33 +764,43 @@ __global__ __launch_bounds__(256) void stk_attn_decode_kernel(StkAttnArgs a) {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int nj = min(64, n_keys - kt0);
+    // the tile's value rows lie in at most two pages: slot of key j = base of its page + offset
     for (int rr = 0; rr < 4; rr++) {
       const int d = lane + 64 * rr;
       if (d >= vdim) break;
       float o = acc[rr] * corr;
-      for (int j = 0; j < nj; j++) {
+      int j = 0;
+      for (; j + 4 <= nj; j += 4) {
+        float v4[4];
+        for (int u = 0; u < 4; u++) {
+          const int kj = kt0 + j + u;
+          v4[u] = El<T>::ld(vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + d);
+        }
+        for (int u = 0; u < 4; u++) o = fmaf(ps[wave * 64 + j + u], v4[u], o);
+      }
+      for (; j < nj; j++) {
         const int kj = kt0 + j;
-        const int64_t slot = (int64_t)bt[kj / a.BS] * a.BS + kj % a.BS;
-        o = fmaf(ps[wave * 64 + j], El<T>::ld(vc + slot * vd_all + g * vdim + d), o);
+        o = fmaf(ps[wave * 64 + j], El<T>::ld(vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + d), o);
       }
       acc[rr] = o;
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
-  if (lane == 0) ms[wave] = m, ms[4 + wave] = l;
+  if (lane == 0) ms[wave] = m, ms[STK_DW + wave] = l;
   for (int rr = 0; rr < 4; rr++) {
     const int d = lane + 64 * rr;
     if (d < vdim) os[wave * vdim + d] = acc[rr];
   }
   __syncthreads();
-  const float M = fmaxf(fmaxf(ms[0], ms[1]), fmaxf(ms[2], ms[3]));
+  float M = ms[0];
+  for (int w = 1; w < STK_DW; w++) M = fmaxf(M, ms[w]);
   T* out = (T*)a.out + (size_t)b * a.H * vdim + h * vdim;
-  for (int d = tid; d < vdim; d += 256) {
+  for (int d = tid; d < vdim; d += 64 * STK_DW) {
     float L = 0.f, o = 0.f;
-    for (int w = 0; w < 4; w++) {
+    for (int w = 0; w < STK_DW; w++) {
       const float c = ms[w] > -INFINITY ? expf(ms[w] - M) : 0.f;
-      L += ms[4 + w] * c;
+      L += ms[STK_DW + w] * c;
       o += os[w * vdim + d] * c;
     }
     El<T>::st(out + d, L > 0.f ? o / L : 0.f);
@@ -590,9 +834,9 @@ void vra_stack_gemm(const StkGemmArgs& g, int dtype, int64_t stream) {
       if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, true><<<grid, 256, 0, st>>>(g); });
       else launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, false><<<grid, 256, 0, st>>>(g); });
     } else {
-      dim3 grid((g.M + 15) / 16, (g.N + 63) / 64);
-      if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<1, 2, 1, 2, true><<<grid, 128, 0, st>>>(g); });
-      else launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<1, 2, 1, 2, false><<<grid, 128, 0, st>>>(g); });
+      dim3 grid((g.M + 15) / 16, (g.N + 31) / 32);
+      if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_small_kernel<true><<<grid, 512, 0, st>>>(g); });
+      else launch_checked("stack gemm", [&] { stk_gemm_mfma_small_kernel<false><<<grid, 512, 0, st>>>(g); });
     }
     return;
   }
@@ -677,11 +921,20 @@ void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream) {
                 "stack attention: heads must be a multiple of kv heads, value size at most 256");
   hipStream_t st = as_stream(stream);
   if (!a.cu_q) {
-    const size_t lds = ((size_t)a.dim + 4 * 64 + 8 + 4 * (size_t)a.vdim) * sizeof(float);
+    const size_t lds = ((size_t)a.dim + STK_DW * 64 + 2 * STK_DW + STK_DW * (size_t)a.vdim) * sizeof(float);
     VRA_CHECK_ARG(lds <= 64 * 1024, "stack attention: head does not fit LDS");
     dim3 grid(a.B, a.H);
-    if (dtype == VRA_F32) launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<float><<<grid, 256, lds, st>>>(a); });
-    else launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<uint16_t><<<grid, 256, lds, st>>>(a); });
+    if (dtype == VRA_F32) launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<float><<<grid, 64 * STK_DW, lds, st>>>(a); });
+    else launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<uint16_t><<<grid, 64 * STK_DW, lds, st>>>(a); });
+    return;
+  }
+  if (dtype == VRA_BF16 && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 256 && a.ldq % 8 == 0 && ((uintptr_t)a.q % 16 == 0)) {
+    dim3 grid((a.max_q + 63) / 64, a.B, a.H);
+#define STK_PFM(DCV, VTV) launch_checked("stack attention (prefill, mfma)", [&] { stk_attn_prefill_mfma_kernel<DCV, VTV><<<grid, 256, 0, st>>>(a); })
+    if (a.dim <= 64 && a.vdim <= 64) STK_PFM(2, 4);
+    else if (a.dim <= 128 && a.vdim <= 128) STK_PFM(4, 8);
+    else STK_PFM(8, 16);
+#undef STK_PFM
     return;
   }
   auto need = [&](int kt) { return ((size_t)STK_QT * a.dim + (size_t)kt * (a.dim + 1) + (size_t)kt * a.vdim + (size_t)STK_QT * kt) * sizeof(float); };

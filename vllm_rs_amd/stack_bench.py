@@ -1,0 +1,124 @@
+"""Throughput of a layer-stack model (Ditilix design) beside the dense bf16 Llama of the same widths — `python bench.py --design ditilix`.
+
+Random weights of layer sizes that resemble a real model; for each size one JSON line with prefill tokens/s (one prompt of
+`prefill_tokens`, best of three engine steps) and decode tokens/s (batches of 1 and 8 behind 512-token prompts, HIP-event time of
+`steps` engine steps), for both models, with the model FLOPs per token and the weight bytes a decode step streams, so that both can be
+priced against the same roofline (2.5 PFLOP/s dense bf16, 8 TB/s).
+"""
+import json
+import time
+
+import numpy as np
+
+
+def stack_config(width, heads, kv_heads, dim, ff, layers, vocab, experts=0, top=2, expert_ff=0, shared_ff=0, share_kv=False):
+    """config.json dict of a Ditilix model: layer 0 dense, the others mixtures of experts when `experts` > 0; with share_kv the second
+    half of the layers reads the keys / values of the last layer of the first half"""
+    mx = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, softcap=50.0, q_temp=dict(coef=0.1, every=1024))
+    ls = []
+    for i in range(layers):
+        m = dict(mx)
+        if share_kv and i >= (layers + 1) // 2:
+            m["kv_from"] = (layers + 1) // 2 - 1
+        if experts and i > 0:
+            mlp = dict(kind="moe", expert=dict(ff=expert_ff, limit=7.0), router=dict(experts=experts, top=top))
+            if shared_ff:
+                mlp["shared"] = dict(ff=shared_ff, limit=7.0)
+        else:
+            mlp = dict(kind="dense", ff=ff)
+        ls.append(dict(type="attention", mixer=m, mlp=mlp))
+    return dict(architecture="Ditilix", width=width, vocab=vocab, residual_mult=0.5, logit_scale=1.0, norm=dict(eps=1e-6, groups=4), layers=ls)
+
+
+def stack_costs(cj):
+    """(matrix FLOPs per token without attention, weight bytes a one-token step reads) of a Ditilix config"""
+    W, flops, wbytes = cj["width"], 0, 0
+    for layer in cj["layers"]:
+        mx, ml = layer["mixer"], layer["mlp"]
+        n = mx["heads"] * mx["dim"] + (0 if mx.get("kv_from") is not None else mx["kv_heads"] * (mx["dim"] + mx["vdim"]))
+        p = W * n + mx["heads"] * mx["vdim"] * W
+        if ml["kind"] == "dense":
+            act = p + 2 * W * ml["ff"]
+        else:
+            act = p + ml["router"]["top"] * 3 * W * ml["expert"]["ff"] + (3 * W * ml["shared"]["ff"] if ml.get("shared") else 0) + W * ml["router"]["experts"]
+        flops += 2 * act
+        wbytes += 2 * act
+    head = cj["vocab"] * W
+    return flops + 2 * head, wbytes + 2 * head
+
+
+def llama_costs(cfg):
+    H, D = cfg["hidden_size"], cfg["head_dim"]
+    per = H * (cfg["num_heads"] + 2 * cfg["num_kv_heads"]) * D + cfg["num_heads"] * D * H + 3 * H * cfg["intermediate_size"]
+    n = per * cfg["num_layers"] + cfg["vocab_size"] * H
+    return 2 * n, 2 * n
+
+
+def measure(eng, L, vocab, prefill_tokens, steps, warmup):
+    def sync():
+        L.vra_device_sync()
+    r = np.random.default_rng(0)
+    best = 1e9
+    for _ in range(3):
+        eng.add_request(r.integers(1, vocab - 1, prefill_tokens).astype(np.uint32), max_tokens=1, ignore_eos=True)
+        sync()
+        t0 = time.perf_counter()
+        eng.step()
+        sync()
+        best = min(best, time.perf_counter() - t0)
+        while eng.has_unfinished():
+            eng.step()
+    out = dict(prefill_tokens_per_s=prefill_tokens / best, prefill_ms=best * 1e3)
+    for bs in (1, 8):
+        for _ in range(bs):
+            eng.add_request(r.integers(1, vocab - 1, 512).astype(np.uint32), max_tokens=warmup + steps + 8, ignore_eos=True)
+        while True:
+            n, is_prefill = eng.step()
+            if not is_prefill and n == bs:
+                break
+        for _ in range(warmup):
+            eng.step()
+        sync()
+        ms = eng.timed_decode(steps)
+        sync()
+        out[f"decode_bs{bs}_tokens_per_s"] = bs * steps / (ms / 1e3)
+        out[f"decode_bs{bs}_ms_per_step"] = ms / steps
+        while eng.has_unfinished():
+            eng.step()
+    return out
+
+
+SIZES = {
+    # name: (width, heads, kv_heads, head size, dense ff, layers, vocab, experts, top, expert ff, shared ff, share_kv)
+    "dense-2048": (2048, 16, 4, 128, 8192, 4, 32000, 0, 0, 0, 0, False),
+    "moe-2048": (2048, 16, 4, 128, 8192, 4, 32000, 16, 2, 1024, 2048, True),
+    "dense-4096": (4096, 32, 8, 128, 14336, 2, 32000, 0, 0, 0, 0, False),
+}
+
+
+def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None):
+    from . import _lib, checkpoint
+    from .engine import BF16, Engine
+    L = _lib.load()
+    lines = []
+    for name in (sizes or SIZES):
+        width, heads, kvh, dim, ff, layers, vocab, experts, top, eff, sff, share = SIZES[name]
+        cj = stack_config(width, heads, kvh, dim, ff, layers, vocab, experts, top, eff, sff, share)
+        eng = Engine(checkpoint.parse_config(cj), num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
+        res = dict(stack=measure(eng, L, vocab, prefill_tokens, steps, warmup))
+        eng.close()
+        res["stack"]["flops_per_token"], res["stack"]["weight_bytes_per_step"] = stack_costs(cj)
+        lcfg = dict(arch="llama", hidden_size=width, intermediate_size=ff, num_layers=layers, num_heads=heads, num_kv_heads=kvh, head_dim=dim,
+                    vocab_size=vocab, max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0, quant_method=None, dtype=BF16)
+        eng = Engine(lcfg, num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
+        res["llama_dense"] = measure(eng, L, vocab, prefill_tokens, steps, warmup)
+        eng.close()
+        res["llama_dense"]["flops_per_token"], res["llama_dense"]["weight_bytes_per_step"] = llama_costs(lcfg)
+        for m in res.values():
+            m["prefill_matrix_tflops"] = m["prefill_tokens_per_s"] * m["flops_per_token"] / 1e12
+            m["decode_bs1_weight_gb_per_s"] = m["weight_bytes_per_step"] / (m["decode_bs1_ms_per_step"] / 1e3) / 1e9
+        line = dict(metric="stack_vs_dense_llama", size=name, design="Ditilix", dtype="bf16", data="synthetic", prefill_tokens=prefill_tokens,
+                    decode_context=512, steps=steps, **res)
+        print(json.dumps(line), flush=True)
+        lines.append(line)
+    return lines

@@ -93,7 +93,17 @@ __global__ __launch_bounds__(256) void stk_group_norm_kernel(StkNormArgs a) {
   const T* rw = (const T*)a.router_w;
   for (int e = wave; e < nz; e += 4) {
     float s = 0.f;
-    for (int c = lane; c < W; c += 64) s = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), s);
+    if (sizeof(T) == 2 && W % 8 == 0 && ((uintptr_t)rw % 16) == 0) {  // 8 weights a load; the lane's partial sums keep one order for a given W
+      for (int c = lane * 8; c < W; c += 64 * 8) {
+        const u32x4 v = *(const u32x4*)((const uint16_t*)rw + (size_t)e * W + c);
+        for (int i = 0; i < 4; i++) {
+          s = fmaf(xs[c + 2 * i], __uint_as_float(v[i] << 16), s);
+          s = fmaf(xs[c + 2 * i + 1], __uint_as_float(v[i] & 0xffff0000u), s);
+        }
+      }
+    } else {
+      for (int c = lane; c < W; c += 64) s = fmaf(xs[c], El<T>::ld(rw + (size_t)e * W + c), s);
+    }
     s = wave_sum(s);
     if (lane == 0) zs[e] = s;
   }
@@ -398,30 +408,38 @@ __global__ __launch_bounds__(256) void stk_gated_act_kernel(const float* gu, T* 
   for (int f = F + threadIdx.x; f < Fp; f += 256) El<T>::st(out + (size_t)m * Fp + f, 0.f);
 }
 
-__device__ __forceinline__ float block_sum256(float v, float* red) {
+#define STK_PN_THREADS 1024
+__device__ __forceinline__ float block_sum_pn(float v, float* red) {
   v = wave_sum(v);
   __syncthreads();
   if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
   __syncthreads();
-  return (red[0] + red[1]) + (red[2] + red[3]);
+  float s = 0.f;
+  for (int w = 0; w < STK_PN_THREADS / 64; w++) s += red[w];
+  return s;
 }
+// one workgroup of 1024 threads per token: up to 8 values per thread stay in registers between the sums and the output
 template <typename T>
-__global__ __launch_bounds__(256) void stk_polynorm_kernel(const float* z, T* out, const float* coef, int F, float eps) {
-  __shared__ float red[4];
+__global__ __launch_bounds__(STK_PN_THREADS) void stk_polynorm_kernel(const float* z, T* out, const float* coef, int F, float eps) {
+  __shared__ float red[STK_PN_THREADS / 64];
   const int m = blockIdx.x;
   const float* zr = z + (size_t)m * F;
+  float keep[8];
   float s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  for (int f = threadIdx.x; f < F; f += 256) {
+  int n = 0;
+  for (int f = threadIdx.x; f < F; f += STK_PN_THREADS, n++) {
     const float v = zr[f], v2 = v * v, v3 = v2 * v;
+    if (n < 8) keep[n] = v;
     s1 = fmaf(v, v, s1), s2 = fmaf(v2, v2, s2), s3 = fmaf(v3, v3, s3);
   }
-  s1 = block_sum256(s1, red);
-  s2 = block_sum256(s2, red);
-  s3 = block_sum256(s3, red);
+  s1 = block_sum_pn(s1, red);
+  s2 = block_sum_pn(s2, red);
+  s3 = block_sum_pn(s3, red);
   const float r1 = 1.f / sqrtf(s1 / (float)F + eps), r2 = 1.f / sqrtf(s2 / (float)F + eps), r3 = 1.f / sqrtf(s3 / (float)F + eps);
   const float ca = coef[0], cb = coef[1], cc = coef[2], ce = coef[3];
-  for (int f = threadIdx.x; f < F; f += 256) {
-    const float v = zr[f], v2 = v * v, v3 = v2 * v;
+  n = 0;
+  for (int f = threadIdx.x; f < F; f += STK_PN_THREADS, n++) {
+    const float v = n < 8 ? keep[n] : zr[f], v2 = v * v, v3 = v2 * v;
     El<T>::st(out + (size_t)m * F + f, ca * (v * r1) + cb * (v2 * r2) + cc * (v3 * r3) + ce);
   }
 }
@@ -459,6 +477,13 @@ __device__ __forceinline__ float q_temperature(int64_t p, float coef, int every)
   return 1.f + coef * logf((float)((p + 1) / every) + 1.f);
 }
 __device__ __forceinline__ float cap_score(float s, float softcap) { return softcap > 0.f ? softcap * tanhf(s / softcap) : s; }
+// the same through the hardware exponential (f32 arithmetic, ~2^-21 relative in the exponential; |error| of the capped score below
+// 2^-22 * softcap): the bf16 kernel's choice, where 16 library calls per lane and key tile would cost more than its matrix products
+__device__ __forceinline__ float cap_score_fast(float s, float softcap) {
+  if (!(softcap > 0.f)) return s;
+  const float x = fminf(fmaxf(s / softcap, -15.f), 15.f);
+  return softcap * (1.f - 2.f / (1.f + __expf(2.f * x)));
+}
 
 // Portions of prompts (and whatever else shares their step): 16 query rows of one head per workgroup, 4 per wave; key tiles of KT
 // tokens staged once in LDS (f32) for all 16 rows; lane = key for the scores, lane = value channel for the weighted sum.
@@ -580,7 +605,8 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
   const int dim = a.dim, vdim = a.vdim;
   const int b = blockIdx.y, h = blockIdx.z, g = h / (a.H / a.G);
   const int q0 = a.cu_q[b], q1 = a.cu_q[b + 1];
-  const int t0 = q0 + blockIdx.x * 64;
+  // the last row blocks of a portion see the most keys: they are dispatched first, so that no long block is left to run alone at the end
+  const int t0 = q0 + ((int)gridDim.x - 1 - (int)blockIdx.x) * 64;
   if (t0 >= q1) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rq = lane & 15, oct = lane >> 4;
   const int tq = t0 + wave * 16 + rq;  // this lane's query row
@@ -612,39 +638,58 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
   f32x4 acc[VT];
   for (int t = 0; t < VT; t++) acc[t] = vra_zero_acc();
   float m = -INFINITY, l = 0.f;
-  for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
-    __syncthreads();
-    // V tile -> LDS, transposed: item = (key, 8 channels)
-    for (int i = tid; i < KT * (VT * 2); i += 256) {
-      const int kl = i / (VT * 2), c8 = (i % (VT * 2)) * 8, key = kt0 + kl;
-      u32x4 v = zero4;
-      if (key < n_keys && c8 < vdim) {
-        const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
-        v = *(const u32x4*)(vc + slot * vd_all + g * vdim + c8);
-      }
-      const int pos = ((kl & 15) >> 2) * 8 + (kl >> 4) * 4 + (kl & 3);
-      for (int e = 0; e < 4; e++) {
-        vt[(c8 + 2 * e) * VLD + pos] = (uint16_t)(v[e] & 0xffffu);
-        vt[(c8 + 2 * e + 1) * VLD + pos] = (uint16_t)(v[e] >> 16);
-      }
-    }
-    __syncthreads();
-    if (kt0 >= n_keys_wave) continue;  // (wave-uniform: nothing of this tile is visible to the wave's rows)
-    // scores of the two 16-key halves
-    f32x4 s[2];
+  // The K fragments and this thread's share of the V tile are requested one tile ahead, so that their way from memory runs beside the
+  // current tile's arithmetic.  V item = (key, 8 channels): NV per thread.
+  constexpr int NV = (KT * VT * 2 + 255) / 256;
+  u32x4 kfn[2][DC], vgn[NV];
+  auto request_tile = [&](int kt0) {
     for (int u = 0; u < 2; u++) {
       const int key = kt0 + u * 16 + rq;
       const bool kv = key < n_keys;
       const int64_t slot = kv ? (int64_t)bt[key / a.BS] * a.BS + key % a.BS : 0;
       const uint16_t* kr = kc + slot * kdim + g * dim;
-      s[u] = vra_zero_acc();
       for (int c = 0; c < DC; c++) {
         const int ch = c * 32 + oct * 8;
         const bool ok = kv && ch < dim;
         const u32x4 kf = *(const u32x4*)(kr + (ok ? ch : 0));
-        const u32x4 kz = ok ? kf : zero4;
-        BF16::mfma(s[u], __builtin_bit_cast(s16x8, kz), __builtin_bit_cast(s16x8, qf[c]));
+        kfn[u][c] = ok ? kf : zero4;
       }
+    }
+    for (int n = 0; n < NV; n++) {
+      const int i = tid + n * 256;
+      const int kl = i / (VT * 2), c8 = (i % (VT * 2)) * 8, key = kt0 + kl;
+      const bool ok = i < KT * VT * 2 && key < n_keys && c8 < vdim;
+      const int64_t slot = ok ? (int64_t)bt[key / a.BS] * a.BS + key % a.BS : 0;
+      const u32x4 v = *(const u32x4*)(vc + slot * vd_all + g * vdim + (ok ? c8 : 0));
+      vgn[n] = ok ? v : zero4;
+    }
+  };
+  request_tile(0);
+  for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
+    u32x4 kfc[2][DC], vgc[NV];
+    for (int u = 0; u < 2; u++)
+      for (int c = 0; c < DC; c++) kfc[u][c] = kfn[u][c];
+    for (int n = 0; n < NV; n++) vgc[n] = vgn[n];
+    __syncthreads();
+    // V tile -> LDS, transposed, the keys in the order the lanes hold their scores
+    for (int n = 0; n < NV; n++) {
+      const int i = tid + n * 256;
+      if (i >= KT * VT * 2) break;
+      const int kl = i / (VT * 2), c8 = (i % (VT * 2)) * 8;
+      const int pos = ((kl & 15) >> 2) * 8 + (kl >> 4) * 4 + (kl & 3);
+      for (int e = 0; e < 4; e++) {
+        vt[(c8 + 2 * e) * VLD + pos] = (uint16_t)(vgc[n][e] & 0xffffu);
+        vt[(c8 + 2 * e + 1) * VLD + pos] = (uint16_t)(vgc[n][e] >> 16);
+      }
+    }
+    __syncthreads();
+    if (kt0 + KT < n_keys) request_tile(kt0 + KT);
+    if (kt0 >= n_keys_wave) continue;  // (wave-uniform: nothing of this tile is visible to the wave's rows)
+    // scores of the two 16-key halves
+    f32x4 s[2];
+    for (int u = 0; u < 2; u++) {
+      s[u] = vra_zero_acc();
+      for (int c = 0; c < DC; c++) BF16::mfma(s[u], __builtin_bit_cast(s16x8, kfc[u][c]), __builtin_bit_cast(s16x8, qf[c]));
     }
     VRA_MFMA_DRAIN();
     float sv[8];
@@ -653,7 +698,7 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
       for (int j = 0; j < 4; j++) {
         const int key = kt0 + u * 16 + oct * 4 + j;
         float x = -INFINITY;
-        if (key <= pq && key < n_keys) x = cap_score(s[u][j] * sc, a.softcap);
+        if (key <= pq && key < n_keys) x = cap_score_fast(s[u][j] * sc, a.softcap);
         sv[u * 4 + j] = x;
         tmax = fmaxf(tmax, x);
       }
@@ -663,9 +708,9 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
     float corr = 1.f, psum = 0.f, pv[8];
     for (int i = 0; i < 8; i++) pv[i] = 0.f;
     if (mn > -INFINITY) {
-      corr = m > -INFINITY ? expf(m - mn) : 0.f;
+      corr = m > -INFINITY ? __expf(m - mn) : 0.f;
       for (int i = 0; i < 8; i++) {
-        pv[i] = sv[i] > -INFINITY ? expf(sv[i] - mn) : 0.f;
+        pv[i] = sv[i] > -INFINITY ? __expf(sv[i] - mn) : 0.f;
         psum += pv[i];
       }
     }
@@ -747,6 +792,12 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
   const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
   const int kdim = a.G * dim, vd_all = a.G * vdim;
   float m = -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+  // 16-bit values in whole octets: the value phase reads 16 bytes a lane (oc = channel octets rounded up to a power of two)
+  const bool vec = sizeof(T) == 2 && vdim % 8 == 0 && ((uintptr_t)vc % 16) == 0;
+  int oc = 1;
+  while (oc * 8 < vdim) oc <<= 1;
+  const int co = lane & (oc - 1), kg = lane / oc, kpar = 64 / oc;
+  float vacc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   for (int kt0 = wave * 64; kt0 < n_keys; kt0 += STK_DW * 64) {
     const int key = kt0 + lane;
     float s = -INFINITY;
@@ -764,34 +815,47 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int nj = min(64, n_keys - kt0);
-    // the tile's value rows lie in at most two pages: slot of key j = base of its page + offset
-    for (int rr = 0; rr < 4; rr++) {
-      const int d = lane + 64 * rr;
-      if (d >= vdim) break;
-      float o = acc[rr] * corr;
-      int j = 0;
-      for (; j + 4 <= nj; j += 4) {
-        float v4[4];
-        for (int u = 0; u < 4; u++) {
-          const int kj = kt0 + j + u;
-          v4[u] = El<T>::ld(vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + d);
-        }
-        for (int u = 0; u < 4; u++) o = fmaf(ps[wave * 64 + j + u], v4[u], o);
-      }
-      for (; j < nj; j++) {
+    if (vec) {
+      // lane = (key group kg, channel octet co): one 16-byte load covers 8 channels of one key, 64 / OC keys are in flight per step;
+      // the groups' partial sums meet after the last tile
+      for (int i = 0; i < 8; i++) vacc[i] *= corr;
+      for (int j = kg; j < nj; j += kpar) {
         const int kj = kt0 + j;
-        o = fmaf(ps[wave * 64 + j], El<T>::ld(vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + d), o);
+        if (co * 8 >= vdim) break;  // (lanes beyond the last octet when the octet count is no power of two)
+        const u32x4 v = *(const u32x4*)((const uint16_t*)vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + co * 8);
+        const float pw = ps[wave * 64 + j];
+        for (int i = 0; i < 4; i++) {
+          vacc[2 * i] = fmaf(pw, __uint_as_float(v[i] << 16), vacc[2 * i]);
+          vacc[2 * i + 1] = fmaf(pw, __uint_as_float(v[i] & 0xffff0000u), vacc[2 * i + 1]);
+        }
       }
-      acc[rr] = o;
+    } else {
+      for (int rr = 0; rr < 4; rr++) {
+        const int d = lane + 64 * rr;
+        if (d >= vdim) break;
+        float o = acc[rr] * corr;
+        for (int j = 0; j < nj; j++) {
+          const int kj = kt0 + j;
+          o = fmaf(ps[wave * 64 + j], El<T>::ld(vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + d), o);
+        }
+        acc[rr] = o;
+      }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
   }
-  if (lane == 0) ms[wave] = m, ms[STK_DW + wave] = l;
-  for (int rr = 0; rr < 4; rr++) {
-    const int d = lane + 64 * rr;
-    if (d < vdim) os[wave * vdim + d] = acc[rr];
+  if (vec) {
+    for (int o = oc; o < 64; o <<= 1)
+      for (int i = 0; i < 8; i++) vacc[i] += __shfl_xor(vacc[i], o, 64);
+    if (lane < oc && co * 8 < vdim)
+      for (int i = 0; i < 8; i++) os[wave * vdim + co * 8 + i] = vacc[i];
+  } else {
+    for (int rr = 0; rr < 4; rr++) {
+      const int d = lane + 64 * rr;
+      if (d < vdim) os[wave * vdim + d] = acc[rr];
+    }
   }
+  if (lane == 0) ms[wave] = m, ms[STK_DW + wave] = l;
   __syncthreads();
   float M = ms[0];
   for (int w = 1; w < STK_DW; w++) M = fmaxf(M, ms[w]);
@@ -889,8 +953,8 @@ void vra_stack_gated_act(const float* gu, void* out, int M, int F, float limit, 
 
 void vra_stack_polynorm(const float* z, void* out, const float* coef, int M, int F, float eps, int dtype, int64_t stream) {
   VRA_CHECK_ARG(z && out && coef && M > 0 && F > 0, "stack polynorm: null pointer or empty shape");
-  if (dtype == VRA_F32) launch_checked("stack polynorm", [&] { stk_polynorm_kernel<float><<<M, 256, 0, as_stream(stream)>>>(z, (float*)out, coef, F, eps); });
-  else launch_checked("stack polynorm", [&] { stk_polynorm_kernel<uint16_t><<<M, 256, 0, as_stream(stream)>>>(z, (uint16_t*)out, coef, F, eps); });
+  if (dtype == VRA_F32) launch_checked("stack polynorm", [&] { stk_polynorm_kernel<float><<<M, STK_PN_THREADS, 0, as_stream(stream)>>>(z, (float*)out, coef, F, eps); });
+  else launch_checked("stack polynorm", [&] { stk_polynorm_kernel<uint16_t><<<M, STK_PN_THREADS, 0, as_stream(stream)>>>(z, (uint16_t*)out, coef, F, eps); });
 }
 
 void vra_stack_residual_combine(float* x, const float* o, const float* p1, int n1, const float* p2, const float* gate, float mult, int T, int W,

@@ -348,20 +348,26 @@ __global__ __launch_bounds__(512) void stk_gemm_mfma_small_kernel(StkGemmArgs g)
   const int k_lo = wave * per * 32, k_hi = min(g.K, (wave + 1) * per * 32);
   f32x4 acc[2] = {vra_zero_acc(), vra_zero_acc()};
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
-  for (int k0 = k_lo; k0 < k_hi; k0 += 32) {
-    const int k = k0 + oct * 8;
-    const bool kin = k < g.K;
-    const int kc = kin ? k : 0;
-    u32x4 af = *(const u32x4*)(ap + kc);
-    if (SCALED) {
-      for (int i = 0; i < 4; i++) af[i] = BF16::pack2(__uint_as_float(af[i] << 16) * asc, __uint_as_float(af[i] & 0xffff0000u) * asc);
+  // four K-steps per round: their twelve 16-byte requests are in flight together, then the eight MFMAs (steps beyond the wave's range
+  // load from offset 0 and count as zeros: same order of the sum, no branch between the MFMAs)
+  for (int k0 = k_lo; k0 < k_hi; k0 += 4 * 32) {
+    u32x4 af[4], wf[4][2];
+    for (int u = 0; u < 4; u++) {
+      const int k = k0 + u * 32 + oct * 8;
+      const bool kin = k < k_hi;
+      const int kc = kin ? k : 0;
+      u32x4 a4 = *(const u32x4*)(ap + kc);
+      if (SCALED) {
+        for (int i = 0; i < 4; i++) a4[i] = BF16::pack2(__uint_as_float(a4[i] << 16) * asc, __uint_as_float(a4[i] & 0xffff0000u) * asc);
+      }
+      af[u] = (idx >= 0 && kin) ? a4 : zero4;
+      for (int nt = 0; nt < 2; nt++) {
+        const u32x4 v = *(const u32x4*)(wp[nt] + kc);
+        wf[u][nt] = (wv[nt] && kin) ? v : zero4;
+      }
     }
-    af = (idx >= 0 && kin) ? af : zero4;
-    for (int nt = 0; nt < 2; nt++) {
-      const u32x4 v = *(const u32x4*)(wp[nt] + kc);
-      const u32x4 wf = (wv[nt] && kin) ? v : zero4;
-      BF16::mfma(acc[nt], __builtin_bit_cast(s16x8, wf), __builtin_bit_cast(s16x8, af));
-    }
+    for (int u = 0; u < 4; u++)
+      for (int nt = 0; nt < 2; nt++) BF16::mfma(acc[nt], __builtin_bit_cast(s16x8, wf[u][nt]), __builtin_bit_cast(s16x8, af[u]));
   }
   VRA_MFMA_DRAIN();
   for (int nt = 0; nt < 2; nt++)
@@ -779,6 +785,7 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
   float* ps = qs + dim;                // [waves][64]
   float* ms = ps + STK_DW * 64;        // [waves] max, [waves] sum
   float* os = ms + 2 * STK_DW;         // [waves][vdim]
+  int* ss = (int*)(os + STK_DW * vdim);  // [waves][64] cache slot of each key of the wave's current tile
   const int b = blockIdx.x, h = blockIdx.y, g = h / (a.H / a.G);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t p = a.positions[b];
@@ -803,6 +810,7 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
     float s = -INFINITY;
     if (key < n_keys) {
       const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
+      ss[wave * 64 + lane] = (int)slot;
       s = cap_score(stk_dot_row<T>(qs, kc + slot * kdim + g * dim, dim) * a.scale, a.softcap);
     }
     const float mn = fmaxf(m, wave_max(s));  // (the tile's first key exists: mn is finite)
@@ -819,25 +827,30 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
       // lane = (key group kg, channel octet co): one 16-byte load covers 8 channels of one key, 64 / OC keys are in flight per step;
       // the groups' partial sums meet after the last tile
       for (int i = 0; i < 8; i++) vacc[i] *= corr;
-      for (int j = kg; j < nj; j += kpar) {
-        const int kj = kt0 + j;
-        if (co * 8 >= vdim) break;  // (lanes beyond the last octet when the octet count is no power of two)
-        const u32x4 v = *(const u32x4*)((const uint16_t*)vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + co * 8);
-        const float pw = ps[wave * 64 + j];
-        for (int i = 0; i < 4; i++) {
-          vacc[2 * i] = fmaf(pw, __uint_as_float(v[i] << 16), vacc[2 * i]);
-          vacc[2 * i + 1] = fmaf(pw, __uint_as_float(v[i] & 0xffff0000u), vacc[2 * i + 1]);
+      // four keys of a group per step, their rows requested together (the slots come from LDS, where the score phase left them, so no
+      // request waits for a block-table read); keys beyond the tile count with weight 0
+      for (int j = kg; j < nj && co * 8 < vdim; j += 4 * kpar) {
+        u32x4 v[4];
+        float pw[4];
+        for (int u = 0; u < 4; u++) {
+          const int ju = j + u * kpar;
+          const bool in = ju < nj;
+          const int64_t sl = ss[wave * 64 + (in ? ju : j)];
+          v[u] = *(const u32x4*)((const uint16_t*)vc + sl * vd_all + g * vdim + co * 8);
+          pw[u] = in ? ps[wave * 64 + ju] : 0.f;
         }
+        for (int u = 0; u < 4; u++)
+          for (int i = 0; i < 4; i++) {
+            vacc[2 * i] = fmaf(pw[u], __uint_as_float(v[u][i] << 16), vacc[2 * i]);
+            vacc[2 * i + 1] = fmaf(pw[u], __uint_as_float(v[u][i] & 0xffff0000u), vacc[2 * i + 1]);
+          }
       }
     } else {
       for (int rr = 0; rr < 4; rr++) {
         const int d = lane + 64 * rr;
         if (d >= vdim) break;
         float o = acc[rr] * corr;
-        for (int j = 0; j < nj; j++) {
-          const int kj = kt0 + j;
-          o = fmaf(ps[wave * 64 + j], El<T>::ld(vc + ((int64_t)bt[kj / a.BS] * a.BS + kj % a.BS) * vd_all + g * vdim + d), o);
-        }
+        for (int j = 0; j < nj; j++) o = fmaf(ps[wave * 64 + j], El<T>::ld(vc + (int64_t)ss[wave * 64 + j] * vd_all + g * vdim + d), o);
         acc[rr] = o;
       }
     }
@@ -985,7 +998,7 @@ void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream) {
                 "stack attention: heads must be a multiple of kv heads, value size at most 256");
   hipStream_t st = as_stream(stream);
   if (!a.cu_q) {
-    const size_t lds = ((size_t)a.dim + STK_DW * 64 + 2 * STK_DW + STK_DW * (size_t)a.vdim) * sizeof(float);
+    const size_t lds = ((size_t)a.dim + 2 * STK_DW * 64 + 2 * STK_DW + STK_DW * (size_t)a.vdim) * sizeof(float);
     VRA_CHECK_ARG(lds <= 64 * 1024, "stack attention: head does not fit LDS");
     dim3 grid(a.B, a.H);
     if (dtype == VRA_F32) launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<float><<<grid, 64 * STK_DW, lds, st>>>(a); });

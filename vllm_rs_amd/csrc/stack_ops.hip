@@ -266,11 +266,12 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
   for (int mt = 0; mt < MT; mt++)
     for (int nt = 0; nt < NT; nt++) acc[mt][nt] = vra_zero_acc();
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
-  for (int k0 = 0; k0 < g.K; k0 += 32) {
+  // the fragments of K-step k + 1 are requested before the MFMAs of step k run
+  u32x4 af[MT], wf[NT], afn[MT], wfn[NT];
+  auto request = [&](int k0, u32x4* ao, u32x4* wo) {
     const int k = k0 + oct * 8;
     const bool kin = k < g.K;
     const int kc = kin ? k : 0;
-    u32x4 af[MT], wf[NT];
     for (int mt = 0; mt < MT; mt++) {
       u32x4 v = *(const u32x4*)(ap[mt] + kc);
       if (SCALED) {
@@ -280,12 +281,18 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
           v[i] = BF16::pack2(lo, hi);
         }
       }
-      af[mt] = (av[mt] && kin) ? v : zero4;
+      ao[mt] = (av[mt] && kin) ? v : zero4;
     }
     for (int nt = 0; nt < NT; nt++) {
       const u32x4 v = *(const u32x4*)(wp[nt] + kc);
-      wf[nt] = (wv[nt] && kin) ? v : zero4;
+      wo[nt] = (wv[nt] && kin) ? v : zero4;
     }
+  };
+  request(0, afn, wfn);
+  for (int k0 = 0; k0 < g.K; k0 += 32) {
+    for (int mt = 0; mt < MT; mt++) af[mt] = afn[mt];
+    for (int nt = 0; nt < NT; nt++) wf[nt] = wfn[nt];
+    request(k0 + 32, afn, wfn);  // (beyond K: loads from offset 0, counted as zeros)
     for (int mt = 0; mt < MT; mt++)
       for (int nt = 0; nt < NT; nt++) BF16::mfma(acc[mt][nt], __builtin_bit_cast(s16x8, wf[nt]), __builtin_bit_cast(s16x8, af[mt]));
   }
@@ -644,15 +651,27 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
   f32x4 acc[VT];
   for (int t = 0; t < VT; t++) acc[t] = vra_zero_acc();
   float m = -INFINITY, l = 0.f;
+  const bool capped = a.softcap > 0.f;
+  const float two_inv_cap = capped ? 2.f / a.softcap : 0.f, two_cap = 2.f * a.softcap;
+  const int key_end = (int)min((int64_t)n_keys, pq + 1);  // this row sees the keys below key_end
   // The K fragments and this thread's share of the V tile are requested one tile ahead, so that their way from memory runs beside the
   // current tile's arithmetic.  V item = (key, 8 channels): NV per thread.
-  constexpr int NV = (KT * VT * 2 + 255) / 256;
-  u32x4 kfn[2][DC], vgn[NV];
-  auto request_tile = [&](int kt0) {
+  // V item = (pair of neighbouring keys, 8 channels): NV per thread, two 16-byte requests each
+  constexpr int NV = (KT / 2 * VT * 2 + 255) / 256;
+  u32x4 kfn[2][DC], vgn[NV][2];
+  // The page size is a multiple of 32 (the launcher sends other sizes to the FMA kernel), so a 32-key tile lies in ONE page: its first
+  // slot is a scalar, read from the block table one tile ahead of the requests that use it — no request of a tile waits behind a
+  // block-table read (vector loads return in order: a per-key read would also wait for everything issued before it).
+  auto page_slot = [&](int kt0) -> int64_t {  // first cache slot of the tile that starts at key kt0 (uniform)
+    const int t = __builtin_amdgcn_readfirstlane(kt0);
+    return t < n_keys ? (int64_t)bt[t / a.BS] * a.BS + t % a.BS : 0;
+  };
+  auto request_tile = [&](int kt0, int64_t slot0) {
+    auto slot_of = [&](int key) { return slot0 + (key - kt0); };
     for (int u = 0; u < 2; u++) {
       const int key = kt0 + u * 16 + rq;
       const bool kv = key < n_keys;
-      const int64_t slot = kv ? (int64_t)bt[key / a.BS] * a.BS + key % a.BS : 0;
+      const int64_t slot = kv ? slot_of(key) : 0;
       const uint16_t* kr = kc + slot * kdim + g * dim;
       for (int c = 0; c < DC; c++) {
         const int ch = c * 32 + oct * 8;
@@ -663,39 +682,51 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
     }
     for (int n = 0; n < NV; n++) {
       const int i = tid + n * 256;
-      const int kl = i / (VT * 2), c8 = (i % (VT * 2)) * 8, key = kt0 + kl;
-      const bool ok = i < KT * VT * 2 && key < n_keys && c8 < vdim;
-      const int64_t slot = ok ? (int64_t)bt[key / a.BS] * a.BS + key % a.BS : 0;
-      const u32x4 v = *(const u32x4*)(vc + slot * vd_all + g * vdim + (ok ? c8 : 0));
-      vgn[n] = ok ? v : zero4;
+      const int kp = i / (VT * 2), c8 = (i % (VT * 2)) * 8;
+      for (int e = 0; e < 2; e++) {
+        const int key = kt0 + kp * 2 + e;
+        const bool ok = i < KT / 2 * VT * 2 && key < n_keys && c8 < vdim;
+        const int64_t slot = ok ? slot_of(key) : 0;
+        const u32x4 v = *(const u32x4*)(vc + slot * vd_all + g * vdim + (ok ? c8 : 0));
+        vgn[n][e] = ok ? v : zero4;
+      }
     }
   };
-  request_tile(0);
+  request_tile(0, page_slot(0));
+  int64_t slot_next = page_slot(KT);
   for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
-    u32x4 kfc[2][DC], vgc[NV];
+    u32x4 kfc[2][DC], vgc[NV][2];
     for (int u = 0; u < 2; u++)
       for (int c = 0; c < DC; c++) kfc[u][c] = kfn[u][c];
-    for (int n = 0; n < NV; n++) vgc[n] = vgn[n];
+    for (int n = 0; n < NV; n++) vgc[n][0] = vgn[n][0], vgc[n][1] = vgn[n][1];
     __syncthreads();
-    // V tile -> LDS, transposed, the keys in the order the lanes hold their scores
+    // V tile -> LDS, transposed, the keys in the order the lanes hold their scores: keys 2 kp and 2 kp + 1 are neighbours there too,
+    // so one 32-bit store carries both for a channel
     for (int n = 0; n < NV; n++) {
       const int i = tid + n * 256;
-      if (i >= KT * VT * 2) break;
-      const int kl = i / (VT * 2), c8 = (i % (VT * 2)) * 8;
-      const int pos = ((kl & 15) >> 2) * 8 + (kl >> 4) * 4 + (kl & 3);
+      if (i >= KT / 2 * VT * 2) break;
+      const int kl = (i / (VT * 2)) * 2, c8 = (i % (VT * 2)) * 8;
+      const int pos = ((kl & 15) >> 2) * 8 + (kl >> 4) * 4 + (kl & 3);  // even
+      uint32_t* row = (uint32_t*)vt;
       for (int e = 0; e < 4; e++) {
-        vt[(c8 + 2 * e) * VLD + pos] = (uint16_t)(vgc[n][e] & 0xffffu);
-        vt[(c8 + 2 * e + 1) * VLD + pos] = (uint16_t)(vgc[n][e] >> 16);
+        const uint32_t lo0 = vgc[n][0][e] & 0xffffu, hi0 = vgc[n][0][e] >> 16, lo1 = vgc[n][1][e] & 0xffffu, hi1 = vgc[n][1][e] >> 16;
+        row[((c8 + 2 * e) * VLD + pos) >> 1] = lo0 | (lo1 << 16);
+        row[((c8 + 2 * e + 1) * VLD + pos) >> 1] = hi0 | (hi1 << 16);
       }
     }
     __syncthreads();
-    if (kt0 + KT < n_keys) request_tile(kt0 + KT);
+    if (kt0 + KT < n_keys) {
+      request_tile(kt0 + KT, slot_next);
+      slot_next = page_slot(kt0 + 2 * KT);
+    }
     if (kt0 >= n_keys_wave) continue;  // (wave-uniform: nothing of this tile is visible to the wave's rows)
     // scores of the two 16-key halves
     f32x4 s[2];
-    for (int u = 0; u < 2; u++) {
-      s[u] = vra_zero_acc();
-      for (int c = 0; c < DC; c++) BF16::mfma(s[u], __builtin_bit_cast(s16x8, kfc[u][c]), __builtin_bit_cast(s16x8, qf[c]));
+    s[0] = vra_zero_acc();
+    s[1] = vra_zero_acc();
+    for (int c = 0; c < DC; c++) {  // (the two halves' chains alternate: an MFMA never waits for the one issued just before it)
+      BF16::mfma(s[0], __builtin_bit_cast(s16x8, kfc[0][c]), __builtin_bit_cast(s16x8, qf[c]));
+      BF16::mfma(s[1], __builtin_bit_cast(s16x8, kfc[1][c]), __builtin_bit_cast(s16x8, qf[c]));
     }
     VRA_MFMA_DRAIN();
     float sv[8];
@@ -703,8 +734,12 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
     for (int u = 0; u < 2; u++)
       for (int j = 0; j < 4; j++) {
         const int key = kt0 + u * 16 + oct * 4 + j;
-        float x = -INFINITY;
-        if (key <= pq && key < n_keys) x = cap_score_fast(s[u][j] * sc, a.softcap);
+        float x = s[u][j] * sc;
+        if (capped) {  // softcap * tanh(x / softcap) = softcap - 2 softcap / (1 + e^(2 x / softcap)), hardware exponential and reciprocal
+          const float y = fminf(fmaxf(x * two_inv_cap, -30.f), 30.f);
+          x = a.softcap - two_cap * __builtin_amdgcn_rcpf(1.f + __expf(y));
+        }
+        x = key < key_end ? x : -INFINITY;
         sv[u * 4 + j] = x;
         tmax = fmaxf(tmax, x);
       }
@@ -732,11 +767,15 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
     for (int t = 0; t < VT; t++) {
       acc[t][0] *= corr, acc[t][1] *= corr, acc[t][2] *= corr, acc[t][3] *= corr;
     }
-    for (int t = 0; t < VT; t++) {
-      const u32x4 vf = *(const u32x4*)(vt + (t * 16 + rq) * VLD + oct * 8);
-      BF16::mfma(acc[t], __builtin_bit_cast(s16x8, vf), __builtin_bit_cast(s16x8, phi));
-      BF16::mfma(acc[t], __builtin_bit_cast(s16x8, vf), __builtin_bit_cast(s16x8, plo));
-    }
+    u32x4 vf[VT];
+#pragma unroll
+    for (int t = 0; t < VT; t++) vf[t] = *(const u32x4*)(vt + (t * 16 + rq) * VLD + oct * 8);
+    // heads of all channel tiles first, then the tails: the two MFMAs into one accumulator are VT instructions apart
+    // (fully unrolled: every accumulator keeps its registers, no indexed register moves next to an MFMA)
+#pragma unroll
+    for (int t = 0; t < VT; t++) BF16::mfma(acc[t], __builtin_bit_cast(s16x8, vf[t]), __builtin_bit_cast(s16x8, phi));
+#pragma unroll
+    for (int t = 0; t < VT; t++) BF16::mfma(acc[t], __builtin_bit_cast(s16x8, vf[t]), __builtin_bit_cast(s16x8, plo));
     VRA_MFMA_DRAIN();
   }
   l += __shfl_xor(l, 16, 64);
@@ -906,7 +945,11 @@ void vra_stack_gemm(const StkGemmArgs& g, int dtype, int64_t stream) {
                     (g.w_group_stride % 8 == 0);
   VRA_CHECK_ARG(g.epi == 0 || (mfma && g.N % 32 == 0), "stack gemm: the gated epilogue needs the bf16 MFMA path and whole gate / up blocks");
   if (mfma) {
-    if (big) {
+    if (big && !g.tile_group && !g.a_scale && g.M >= 256 && (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) >= 256) {
+      // enough 128 x 128 tiles to fill the chip: a wave owns 64 x 64 (16 MFMAs per 8 fragment requests instead of 8 per 6)
+      dim3 grid((g.M + 127) / 128, (g.N + 127) / 128);
+      launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<4, 4, 2, 2, false><<<grid, 256, 0, st>>>(g); });
+    } else if (big) {
       dim3 grid((g.M + 63) / 64, (g.N + 127) / 128);
       if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, true><<<grid, 256, 0, st>>>(g); });
       else launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, false><<<grid, 256, 0, st>>>(g); });
@@ -1005,7 +1048,7 @@ void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream) {
     else launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<uint16_t><<<grid, 64 * STK_DW, lds, st>>>(a); });
     return;
   }
-  if (dtype == VRA_BF16 && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 256 && a.ldq % 8 == 0 && ((uintptr_t)a.q % 16 == 0)) {
+  if (dtype == VRA_BF16 && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 256 && a.ldq % 8 == 0 && ((uintptr_t)a.q % 16 == 0) && a.BS % 32 == 0) {
     dim3 grid((a.max_q + 63) / 64, a.B, a.H);
 #define STK_PFM(DCV, VTV) launch_checked("stack attention (prefill, mfma)", [&] { stk_attn_prefill_mfma_kernel<DCV, VTV><<<grid, 256, 0, st>>>(a); })
     if (a.dim <= 64 && a.vdim <= 64) STK_PFM(2, 4);

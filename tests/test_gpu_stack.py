@@ -111,7 +111,8 @@ def config_a():
         dict(type="attention", mixer=mixer(), mlp=moe()),
         dict(type="attention", mixer=mixer(kv_from=1), mlp=moe(shared=None)),
         dict(type="attention", mixer=mixer(kv_from=1, softcap=0, q_temp=None), mlp=None),
-        dict(type="attention", mixer=mixer(heads=4, kv_heads=4, dim=8, vdim=8, scale=0.5, softcap=0, q_temp=(0.5, 64)), mlp=dict(kind="dense", ff=16)),
+        # (key size a multiple of 8, value size a multiple of 16: the bf16 model runs this layer's prompt portions on the matrix-core kernel)
+        dict(type="attention", mixer=mixer(heads=4, kv_heads=4, dim=24, vdim=16, scale=0.5, softcap=4.0, q_temp=(0.5, 64)), mlp=dict(kind="dense", ff=16)),
     ])
 
 
@@ -340,7 +341,8 @@ def run_attention(L, q, positions, k, v, mx, dt, decode, r, BS=64):
 
 @pytest.mark.parametrize("dt", [F32, BF16])
 @pytest.mark.parametrize("decode", [False, True])
-@pytest.mark.parametrize("H,G,dim,vdim", [(6, 3, 16, 24), (4, 4, 8, 8), (2, 1, 5, 7), (8, 2, 128, 128), (3, 1, 40, 200)])
+@pytest.mark.parametrize("H,G,dim,vdim", [(6, 3, 16, 24), (4, 4, 8, 8), (2, 1, 5, 7), (8, 2, 128, 128), (3, 1, 40, 200), (6, 2, 32, 48), (4, 2, 64, 16),
+                                          (2, 1, 160, 144), (5, 5, 72, 80)])
 def test_attention_random(dt, decode, H, G, dim, vdim):
     L = _lib.load()
     r = np.random.default_rng(H * 100 + dim)
@@ -364,7 +366,8 @@ def test_attention_planted_key(dt, decode, softcap, temp):
     key is already in the cache, as in a prompt's portion)."""
     L = _lib.load()
     r = np.random.default_rng(11)
-    Tk, H, G, dim, vdim = 900, 4, 2, 16, 8
+    Tk, H, G = 900, 4, 2
+    dim, vdim = (32, 16) if temp else (16, 8)  # (the first pair runs the bf16 prompt form on the matrix-core kernel, the second on FMA)
     mx = dict(scale=0.25, softcap=softcap)
     if temp:
         mx["q_temp"] = temp
@@ -385,7 +388,7 @@ def test_attention_planted_key(dt, decode, softcap, temp):
             if p >= j:
                 assert np.abs(got[i] - 5.0).max() < 0.05, (j, p)
             else:
-                assert np.abs(got[i]).max() < 0.2, (j, p)
+                assert np.abs(got[i]).max() < 0.6, (j, p)  # (the other values are 0.1 N(0, 1); the marker is 5)
 
 
 # ------------------------------------------------------------------------------------------------ whole models through the engine

@@ -250,6 +250,7 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
   const uint16_t* wp[NT];
   bool av[MT], wv[NT];
   float asc[MT];
+#pragma unroll
   for (int mt = 0; mt < MT; mt++) {
     const int r = m_base + mt * 16 + rq;
     const int idx = r < g.M ? (g.a_row ? g.a_row[r] : r) : -1;
@@ -257,13 +258,16 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
     ap[mt] = A + (int64_t)(idx >= 0 ? idx : 0) * g.lda;
     asc[mt] = SCALED && idx >= 0 ? g.a_scale[r] : 1.f;
   }
+#pragma unroll
   for (int nt = 0; nt < NT; nt++) {
     const int n = n_base + nt * 16 + rq;
     wv[nt] = n < g.N;
     wp[nt] = Wt + (int64_t)(n < g.N ? n : 0) * g.K;
   }
   f32x4 acc[MT][NT];
+#pragma unroll
   for (int mt = 0; mt < MT; mt++)
+#pragma unroll
     for (int nt = 0; nt < NT; nt++) acc[mt][nt] = vra_zero_acc();
   const u32x4 zero4 = {0u, 0u, 0u, 0u};
   // the fragments of K-step k + 1 are requested before the MFMAs of step k run
@@ -272,7 +276,8 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
     const int k = k0 + oct * 8;
     const bool kin = k < g.K;
     const int kc = kin ? k : 0;
-    for (int mt = 0; mt < MT; mt++) {
+  #pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
       u32x4 v = *(const u32x4*)(ap[mt] + kc);
       if (SCALED) {
         const float s = asc[mt];
@@ -283,27 +288,34 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
       }
       ao[mt] = (av[mt] && kin) ? v : zero4;
     }
-    for (int nt = 0; nt < NT; nt++) {
+  #pragma unroll
+  for (int nt = 0; nt < NT; nt++) {
       const u32x4 v = *(const u32x4*)(wp[nt] + kc);
       wo[nt] = (wv[nt] && kin) ? v : zero4;
     }
   };
   request(0, afn, wfn);
   for (int k0 = 0; k0 < g.K; k0 += 32) {
+#pragma unroll
     for (int mt = 0; mt < MT; mt++) af[mt] = afn[mt];
+#pragma unroll
     for (int nt = 0; nt < NT; nt++) wf[nt] = wfn[nt];
     request(k0 + 32, afn, wfn);  // (beyond K: loads from offset 0, counted as zeros)
+#pragma unroll
     for (int mt = 0; mt < MT; mt++)
+#pragma unroll
       for (int nt = 0; nt < NT; nt++) BF16::mfma(acc[mt][nt], __builtin_bit_cast(s16x8, wf[nt]), __builtin_bit_cast(s16x8, af[mt]));
   }
   VRA_MFMA_DRAIN();
   // lane: activation row rq of tile mt, output columns oct * 4 + j of tile nt
+#pragma unroll
   for (int mt = 0; mt < MT; mt++) {
     const int r = m_base + mt * 16 + rq;
     if (r >= g.M || !av[mt]) continue;
     const int orow = g.out_row ? g.out_row[r] : r;
     if (orow < 0) continue;
     if (g.epi == 1) {
+#pragma unroll
       for (int nt = 0; nt + 1 < NT; nt += 2)
         for (int j = 0; j < 4; j++) {
           const int n = (n_base + nt * 16) / 2 + oct * 4 + j;
@@ -313,6 +325,7 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
           else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(y);
         }
     } else {
+#pragma unroll
       for (int nt = 0; nt < NT; nt++)
         for (int j = 0; j < 4; j++) {
           const int n = n_base + nt * 16 + oct * 4 + j;
@@ -439,10 +452,15 @@ __global__ __launch_bounds__(STK_PN_THREADS) void stk_polynorm_kernel(const floa
   const float* zr = z + (size_t)m * F;
   float keep[8];
   float s1 = 0.f, s2 = 0.f, s3 = 0.f;
-  int n = 0;
-  for (int f = threadIdx.x; f < F; f += STK_PN_THREADS, n++) {
+#pragma unroll
+  for (int n = 0; n < 8; n++) {  // the first 8192 values: one per thread and round, kept in registers
+    const int f = threadIdx.x + n * STK_PN_THREADS;
+    const float v = f < F ? zr[f] : 0.f, v2 = v * v, v3 = v2 * v;
+    keep[n] = v;
+    s1 = fmaf(v, v, s1), s2 = fmaf(v2, v2, s2), s3 = fmaf(v3, v3, s3);
+  }
+  for (int f = threadIdx.x + 8 * STK_PN_THREADS; f < F; f += STK_PN_THREADS) {
     const float v = zr[f], v2 = v * v, v3 = v2 * v;
-    if (n < 8) keep[n] = v;
     s1 = fmaf(v, v, s1), s2 = fmaf(v2, v2, s2), s3 = fmaf(v3, v3, s3);
   }
   s1 = block_sum_pn(s1, red);
@@ -450,9 +468,14 @@ __global__ __launch_bounds__(STK_PN_THREADS) void stk_polynorm_kernel(const floa
   s3 = block_sum_pn(s3, red);
   const float r1 = 1.f / sqrtf(s1 / (float)F + eps), r2 = 1.f / sqrtf(s2 / (float)F + eps), r3 = 1.f / sqrtf(s3 / (float)F + eps);
   const float ca = coef[0], cb = coef[1], cc = coef[2], ce = coef[3];
-  n = 0;
-  for (int f = threadIdx.x; f < F; f += STK_PN_THREADS, n++) {
-    const float v = n < 8 ? keep[n] : zr[f], v2 = v * v, v3 = v2 * v;
+#pragma unroll
+  for (int n = 0; n < 8; n++) {
+    const int f = threadIdx.x + n * STK_PN_THREADS;
+    const float v = keep[n], v2 = v * v, v3 = v2 * v;
+    if (f < F) El<T>::st(out + (size_t)m * F + f, ca * (v * r1) + cb * (v2 * r2) + cc * (v3 * r3) + ce);
+  }
+  for (int f = threadIdx.x + 8 * STK_PN_THREADS; f < F; f += STK_PN_THREADS) {
+    const float v = zr[f], v2 = v * v, v3 = v2 * v;
     El<T>::st(out + (size_t)m * F + f, ca * (v * r1) + cb * (v2 * r2) + cc * (v3 * r3) + ce);
   }
 }
@@ -584,6 +607,7 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
     for (int rr = 0; rr < 4; rr++) {
       const int d = lane + 64 * rr;
       if (d >= vdim) break;
+#pragma unroll 4
       for (int j = 0; j < KT; j++) {
         const float v = vs[j * vdim + d];
         for (int i = 0; i < 4; i++) acc[i][rr] = fmaf(ps[(wave * 4 + i) * KT + j], v, acc[i][rr]);

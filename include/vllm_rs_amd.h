@@ -425,7 +425,7 @@ typedef struct vra_model_config {
 
 /* vra_model_config.arch of a model that is a LIST OF LAYERS (vllm_rs_amd/host/stack_model.h): hidden_size = width, vocab_size, num_layers,
  * dtype (VRA_BF16 or VRA_F32) and max_position_embeddings are read from the struct, everything else from the spec text of
- * vra_engine_create_spec.  The Ditilix design loads as such a model. */
+ * vra_engine_create_spec.  The Ditilix and Gaperax designs load as such models. */
 #define VRA_ARCH_STACK 3
 
 typedef struct vra_engine_config {
@@ -650,6 +650,35 @@ void vra_stack_op_attention(const void* q, int32_t ldq, void* out, const void* k
                             const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
                             int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks,
                             float scale, float softcap, float temp_coef, int32_t temp_every, int32_t dtype, int64_t stream);
+
+/* more operators of layer-stack models: sequential pre-norm blocks with a Dynamic Tanh norm, latent (low-rank) attention with a rotary
+ * part and a softmax sink, attention with sigmoid weights / distance penalty / window / mixed heads / output gate
+ * (vllm_rs_amd/csrc/stack_launch.h states each) */
+void vra_stack_op_dyt(float* x, const float* add, const float* w, const float* b, float alpha, void* h, int32_t T, int32_t W,
+                      int32_t dtype, int64_t stream);
+void vra_stack_op_latent_prep(const float* raw, int32_t ld, int32_t q_rank, int32_t kv_rank, int32_t rot_dim, const float* qn_w,
+                              const float* kvn_w, float eps, void* cq, void* cache, int32_t cache_ld, const int64_t* slots,
+                              const int64_t* positions, const float* freq_hi, const float* freq_lo, int32_t pairs, float mag,
+                              int32_t T, int32_t dtype, int64_t stream);
+void vra_stack_op_rope_heads(const void* in, int32_t in_ld, int32_t in_hs, int32_t in_off, void* out, int32_t out_ld, int32_t out_hs,
+                             int32_t out_off, int32_t n, int32_t H, const int64_t* positions, const float* freq_hi,
+                             const float* freq_lo, int32_t pairs, float mag, int32_t T, int32_t dtype, int64_t stream);
+void vra_stack_op_qk_norm_store(const float* raw, int32_t ld, int32_t nq, int32_t nk, int32_t nv, const float* q_w, const float* k_w,
+                                float eps, void* q_out, void* kc, void* vc, const int64_t* slots, int32_t T, int32_t dtype,
+                                int64_t stream);
+void vra_stack_op_sigmoid_attention(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                    const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B,
+                                    int32_t T, int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS,
+                                    int32_t max_blocks, float scale, int32_t window, int32_t keep_first, const float* slopes,
+                                    const float* head_bias, const float* talk, const float* gate, int32_t gate_ld, int32_t dtype,
+                                    int64_t stream);
+void vra_stack_op_gemm_ex(const void* a, int32_t lda, const void* w, void* out, int32_t ldo, int32_t out_f32, int32_t M, int32_t N,
+                          int32_t K, float alpha, const float* bias, int32_t epi, int32_t act, int32_t batch, int64_t a_batch_stride,
+                          int64_t w_batch_stride, int64_t out_batch_stride, int32_t dtype, int64_t stream);
+void vra_stack_op_attention_ex(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                               const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                               int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks,
+                               float scale, const float* sink, int32_t k_ld, int32_t v_ld, int32_t dtype, int64_t stream);
 
 /* decode-step microbenchmark hook used by bench.py: runs `steps` decode steps of the current
  * running batch back to back (graph replay when enabled) and returns elapsed ms measured with HIP

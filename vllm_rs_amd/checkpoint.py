@@ -98,7 +98,54 @@ def parse_ditilix(cfg_json, dtype=None):
                 rms_norm_eps=float(norm.get("eps", 1e-6)), rope_theta=10000.0, dtype=dt, quant_method=None, spec="\n".join(lines) + "\n")
 
 
-STACK_ARCHS = {"Ditilix": parse_ditilix}
+def parse_gaperax(cfg_json, dtype=None):
+    """Gaperax config.json -> cfg dict with arch "stack": sequential pre-norm blocks with a Dynamic Tanh norm, no position vector at the
+    embedding, and per layer a latent attention (low-rank latents, rotary part with optional YaRN scaling, softmax sink) or an attention
+    with sigmoid weights (distance penalty, window with kept first tokens, mixed heads, output gate), a gated gelu feed-forward or none,
+    optionally the tensors of another layer ("weights_of").  Every size and constant comes from the config."""
+    td = dtype or cfg_json.get("torch_dtype", "bfloat16")
+    dt = {"bfloat16": BF16, "bf16": BF16, "float32": F32, "f32": F32, BF16: BF16, F32: F32}.get(td)
+    if dt is None:
+        raise ValueError(f"dtype {td!r}: a layer stack runs in bfloat16 or float32")
+    norm = cfg_json.get("norm") or {}
+    width, vocab, layers = int(cfg_json["width"]), int(cfg_json["vocab"]), cfg_json["layers"]
+    lines = ["stack width=%d vocab=%d eps=%s block=sequential norm=dyt pos=none" % (width, vocab, _num(norm.get("eps", 1e-6)))]
+    heads = kv_heads = dim = 1
+    for i, layer in enumerate(layers):
+        mx, kind = layer["mixer"], layer.get("type")
+        f = dict(heads=int(mx["heads"]), dim=int(mx["dim"]), vdim=int(mx.get("vdim", mx["dim"])),
+                 scale=_num(mx["scale"]) if mx.get("scale") is not None else _num(int(mx["dim"]) ** -0.5))
+        if kind == "latent_attention":
+            rot = mx.get("rot") or {}
+            f.update(mixer="latent", kv_heads=1, rot_dim=int(mx.get("rot_dim", 0)), kv_rank=int(mx["kv_rank"]), q_rank=int(mx["q_rank"]), sink=1,
+                     rot_dims=int(rot.get("dims", mx.get("rot_dim", 0))), rot_base=_num(rot.get("base", 10000.0)))
+            sc = rot.get("scaling")
+            if sc:
+                f.update(yarn_factor=_num(sc["factor"]), yarn_original=_num(sc["original"]), yarn_fast=_num(sc.get("fast", 32.0)),
+                         yarn_slow=_num(sc.get("slow", 1.0)))
+        elif kind == "attention":
+            mask = mx.get("mask") or {}
+            f.update(mixer="sigmoid", kv_heads=int(mx.get("kv_heads", mx["heads"])), window=int(mask.get("size", 0)),
+                     keep_first=int(mask.get("keep_first", 0)), slope_exp=_num(8.0))
+        else:
+            raise ValueError(f"layer {i}: mixer type {kind!r} is not part of this design")
+        if layer.get("weights_of") is not None:
+            f.update(weights_of=int(layer["weights_of"]))
+        mlp = layer.get("mlp")
+        if not mlp:
+            f.update(mlp="none")
+        elif mlp["kind"] == "dense":
+            f.update(mlp="gated", ff=int(mlp["ff"]))
+        else:
+            raise ValueError(f"layer {i}: feed-forward kind {mlp['kind']!r} is not part of this design")
+        lines.append("layer " + " ".join(f"{k}={v}" for k, v in f.items()))
+        heads, kv_heads, dim = max(heads, f["heads"]), max(kv_heads, f["kv_heads"]), max(dim, f["dim"], f["vdim"])
+    return dict(arch="stack", design="Gaperax", hidden_size=width, vocab_size=vocab, num_layers=len(layers), num_heads=heads, num_kv_heads=kv_heads,
+                head_dim=dim, intermediate_size=0, max_position_embeddings=int(cfg_json.get("max_position_embeddings", 1 << 20)),
+                rms_norm_eps=float(norm.get("eps", 1e-6)), rope_theta=10000.0, dtype=dt, quant_method=None, spec="\n".join(lines) + "\n")
+
+
+STACK_ARCHS = {"Ditilix": parse_ditilix, "Gaperax": parse_gaperax}
 
 
 def parse_config(cfg_json, dtype=None):

@@ -728,6 +728,7 @@ extern "C" void vra_cast(const void* in, void* out, int64_t numel, int32_t in_dt
 extern "C" void vra_swap_blocks(const void* src, void* dst, const int64_t* h_pairs, int32_t n_pairs, int64_t block_bytes,
                                 int32_t kind, int64_t stream) {
   hipMemcpyKind mk = kind == 0 ? hipMemcpyDeviceToDevice : (kind == 1 ? hipMemcpyDeviceToHost : hipMemcpyHostToDevice);
+  if (block_bytes <= 0) return;  // (a cache without blocks of this kind)
   for (int i = 0; i < n_pairs; i++) {
     const char* s = static_cast<const char*>(src) + h_pairs[2 * i] * block_bytes;
     char* d = static_cast<char*>(dst) + h_pairs[2 * i + 1] * block_bytes;

@@ -1,0 +1,40 @@
+// stack_common.cuh — helpers shared by the operator files of config-driven layer stacks (stack_ops.hip, stack_mixers.hip).
+#pragma once
+#include <math.h>
+
+#include "common.cuh"
+
+namespace {
+
+template <typename T>
+struct El;
+template <>
+struct El<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float rnd(float v) { return v; }
+};
+template <>
+struct El<uint16_t> {
+  static __device__ __forceinline__ float ld(const uint16_t* p) { return BF16::to_f32(*p); }
+  static __device__ __forceinline__ void st(uint16_t* p, float v) { *p = BF16::from_f32(v); }
+  static __device__ __forceinline__ float rnd(float v) { return BF16::to_f32(BF16::from_f32(v)); }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
+template <typename F>
+void launch_checked(const char* what, F f) {
+  f();
+  const hipError_t e = hipGetLastError();
+  if (e != hipSuccess) vra_set_error("%s: %s", what, hipGetErrorString(e));
+}
+
+}  // namespace

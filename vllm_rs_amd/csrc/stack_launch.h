@@ -30,12 +30,19 @@ struct StkGemmArgs {
   const int* out_row = nullptr;
   int epi = 0;
   float limit = 0.f, act_alpha = 1.702f;
+  int act = 0;                  // the gated pair of epi 1: 0 the clamped form above, 1  gelu_tanh(g) * u
+  const float* bias = nullptr;  // f32 [N], added after alpha (plain epilogue)
+  // batched form (no row groups): product z of `batch` reads a + z * a_batch_stride, w + z * w_batch_stride and writes out + z * out_batch_stride
+  // (element counts; a column offset per head turns one launch into a product per head)
+  int batch = 1;
+  int64_t a_batch_stride = 0, w_batch_stride = 0, out_batch_stride = 0;
 };
 void vra_stack_gemm(const StkGemmArgs& g, int dtype, int64_t stream);
 // rows per granule the grouped launches of an M-row problem over `groups` groups want (16 or 64)
 int vra_stack_gemm_granule(int rows, int groups);
 
-// x[t, c] = embed[ids[t], c] + pe(positions[t], c),  pe(p, 2i) = sin(p * inv_freq[i]),  pe(p, 2i+1) = cos(p * inv_freq[i])  (f32)
+// x[t, c] = embed[ids[t], c] + pe(positions[t], c),  pe(p, 2i) = sin(p * inv_freq[i]),  pe(p, 2i+1) = cos(p * inv_freq[i])  (f32);
+// inv_freq null: no position vector
 void vra_stack_embed_sinpos(const uint32_t* ids, const int64_t* positions, const void* embed, const float* inv_freq, float* x, int T, int W, int V,
                             int dtype, int64_t stream);
 
@@ -63,7 +70,7 @@ void vra_stack_moe_sort(const int* pair_expert, const float* pair_weight, int P,
                         float* row_scale, int* row_pair, int* tile_group, int64_t stream);
 
 // the gated pair of epi 1 on an f32 [M, 2 * F] matrix whose column blocks of 16 alternate gate / up -> out [M, F] in dtype
-void vra_stack_gated_act(const float* gu, void* out, int M, int F, float limit, float act_alpha, int dtype, int64_t stream);
+void vra_stack_gated_act(const float* gu, void* out, int M, int F, float limit, float act_alpha, int dtype, int64_t stream, int act = 0);
 
 // PolyNorm: out = a N(z) + b N(z^2) + c N(z^3) + e,  N(v) = v / sqrt(mean(v^2) + eps) over a token's F values; coef = {a, b, c, e} (device, f32)
 void vra_stack_polynorm(const float* z, void* out, const float* coef, int M, int F, float eps, int dtype, int64_t stream);
@@ -93,8 +100,83 @@ struct StkAttnArgs {
   int B = 0, T = 0, max_q = 1, H = 0, G = 0, dim = 0, vdim = 0, BS = 64, max_blocks = 0;
   float scale = 1.f, softcap = 0.f, temp_coef = 0.f;
   int temp_every = 0;
+  const float* sink = nullptr;  // f32 [H]: the softmax denominator also holds exp(sink[h]) — a term without key or value, counted once
+  int k_ld = 0, v_ld = 0;       // elements between the rows of kc / vc (0: G * dim / G * vdim).  A latent cache keeps one row [c | rotated
+                                // part] per token: keys are the whole row, values its first columns (vc = kc, v_ld = k_ld)
 };
 void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream);
 
 // rows of a [*, W] f32 matrix picked by index -> dst (f32)
 void vra_stack_gather_rows_f32(const float* src, const uint32_t* rows, float* dst, int n, int W, int64_t stream);
+
+// ---------------------------------------------------------------------------------------------------------------------------------------
+// Operators of sequential pre-norm blocks with other mixers (stack_mixers.hip)
+
+// Dynamic Tanh "norm" with the residual sum folded in:  x += add (add null: x as it is);  h = tanh(alpha * x) * w + b   (x, add, w, b f32;
+// h in dtype).  No statistics of the row.
+void vra_stack_dyt(float* x, const float* add, const float* w, const float* b, float alpha, void* h, int T, int W, int dtype, int64_t stream);
+
+// Rotary angles: pair i of a vector at position p turns by p * (freq_hi[i] + freq_lo[i]) (the frequency as an unevaluated sum of two f32,
+// so that the f32 angle carries no rounding of the frequency); (u, v) -> mag * (u cos - v sin, v cos + u sin); the pair is (2i, 2i + 1).
+struct StkRotary {
+  const float* freq_hi = nullptr;
+  const float* freq_lo = nullptr;
+  int pairs = 0;      // rotated dimensions / 2; the dimensions behind them pass unchanged
+  float mag = 1.f;    // multiplies cos and sin
+};
+
+// Latent projections of one token, from the f32 row  raw = [a | b | r]  of the joint down-projection:
+//   cq = rmsnorm(a) * qn_w                      -> cq [T, q_rank] in dtype
+//   c  = rmsnorm(b) * kvn_w, rot(r) at position -> cache row [c | rot(r)] at the token's slot (cache_ld elements per row; slot < 0: skipped)
+// rmsnorm(v) = v / sqrt(mean(v^2) + eps).
+struct StkLatentPrepArgs {
+  const float* raw = nullptr;
+  int ld = 0, q_rank = 0, kv_rank = 0, rot_dim = 0;
+  const float* qn_w = nullptr;
+  const float* kvn_w = nullptr;
+  float eps = 1e-6f;
+  void* cq = nullptr;
+  void* cache = nullptr;
+  int cache_ld = 0;
+  const int64_t* slots = nullptr;
+  const int64_t* positions = nullptr;
+  StkRotary rot;
+  int T = 0;
+};
+void vra_stack_latent_prep(const StkLatentPrepArgs& a, int dtype, int64_t stream);
+
+// Rotary on the rows of a head-by-head matrix: for every token t and head h the `n` values at in[t, h * in_hs + in_off ..] are rotated at
+// positions[t] and written to out[t, h * out_hs + out_off ..] (both in dtype; in == out allowed when the ranges are the same).
+void vra_stack_rope_heads(const void* in, int in_ld, int in_hs, int in_off, void* out, int out_ld, int out_hs, int out_off, int n, int H,
+                          const int64_t* positions, const StkRotary& rot, int T, int dtype, int64_t stream);
+
+// One RMS norm over ALL of q and one over ALL of k (before the split into heads), from the f32 row  raw = [q | k | v | ...]:
+//   q_out = rmsnorm(q) * q_w (dtype) ; cache K row = rmsnorm(k) * k_w ; cache V row = v   (q_w / k_w null: that norm is skipped)
+void vra_stack_qk_norm_store(const float* raw, int ld, int nq, int nk, int nv, const float* q_w, const float* k_w, float eps, void* q_out, void* kc,
+                             void* vc, const int64_t* slots, int T, int dtype, int64_t stream);
+
+// Attention without softmax over the paged cache: every visible key j of query i (positions p_i, j) weighs
+//   w_h(i, j) = sigmoid((q_h . k_g) * scale - slopes[h] * (p_i - j) + head_bias[h]),   visible: j <= p_i and (p_i - j < window or j < keep_first)
+// (window <= 0: every j <= p_i), not normalised over keys; the heads' weights are mixed, w'_h = sum_g talk[h, g] w_g; head h applies w'_h to
+// the values of its own key/value head; the output row is multiplied by sigmoid(gate) element by element.  slopes, head_bias, talk, gate
+// null: that term is absent.  Scores, weights and sums f32; keys are summed in ascending order in tiles aligned to absolute positions.
+struct StkSigAttnArgs {
+  const void* q = nullptr;
+  int ldq = 0;
+  void* out = nullptr;  // [T, H * vdim] in dtype
+  const void* kc = nullptr;
+  const void* vc = nullptr;
+  const int64_t* positions = nullptr;
+  const uint32_t* block_tables = nullptr;
+  const uint32_t* context_lens = nullptr;
+  const uint32_t* cu_q = nullptr;  // prefill form [B + 1]; null: one token per sequence
+  int B = 0, T = 0, max_q = 1, H = 0, G = 0, dim = 0, vdim = 0, BS = 64, max_blocks = 0;
+  float scale = 1.f;
+  int window = 0, keep_first = 0;
+  const float* slopes = nullptr;     // [H]
+  const float* head_bias = nullptr;  // [H]
+  const float* talk = nullptr;       // [H, H]
+  const float* gate = nullptr;       // f32 [T, gate_ld], H * vdim columns used
+  int gate_ld = 0;
+};
+void vra_stack_sigmoid_attention(const StkSigAttnArgs& a, int dtype, int64_t stream);

@@ -1,0 +1,399 @@
+// stack_mixers.hip — operators of sequential pre-norm layer stacks (host/stack_model.cpp; each is specified in stack_launch.h), gfx950:
+// Dynamic Tanh with the residual sum, the latent (low-rank) attention's norms / rotary / cache rows, the whole-projection query / key norm,
+// and the attention without softmax (sigmoid weights, distance penalty, window with kept first tokens, mixed heads, output gate).
+//
+// f32 whatever the storage type: positions and angles, norms, scores and weights, every sum over keys.  The order of every sum depends
+// on the model's shapes and on absolute positions alone, never on the step's rows, so a token's result does not depend on how its
+// prompt was cut or on its batch.
+#include <algorithm>
+
+#include "stack_common.cuh"
+#include "stack_launch.h"
+
+namespace {
+
+__device__ __forceinline__ float block_sum_256(float v, float* red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return (red[0] + red[1]) + (red[2] + red[3]);
+}
+
+// cos / sin of p * (hi + lo), times mag: the product p * hi is split exactly (fma), the small part enters to first order
+__device__ __forceinline__ void rot_cos_sin(const StkRotary& r, int i, float p, float* c, float* s) {
+  const float fh = r.freq_hi[i], fl = r.freq_lo ? r.freq_lo[i] : 0.f;
+  const float ah = p * fh;
+  const float al = fmaf(p, fh, -ah) + p * fl;
+  const float c0 = cosf(ah), s0 = sinf(ah);
+  *c = (c0 - s0 * al) * r.mag;
+  *s = (s0 + c0 * al) * r.mag;
+}
+
+// ------------------------------------------------------------------------------------------------ Dynamic Tanh (+ residual sum)
+template <typename T>
+__global__ __launch_bounds__(256) void stk_dyt_kernel(float* x, const float* add, const float* w, const float* b, float alpha, T* h, int W, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+    const int c = (int)(i % W);
+    float v = x[i];
+    if (add) {
+      v += add[i];
+      x[i] = v;
+    }
+    El<T>::st(h + i, tanhf(alpha * v) * w[c] + b[c]);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ latent attention: norms, rotary, cache row
+template <typename T>
+__global__ __launch_bounds__(256) void stk_latent_prep_kernel(StkLatentPrepArgs a) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float* raw = a.raw + (size_t)t * a.ld;
+  float s = 0.f;
+  for (int c = tid; c < a.q_rank; c += 256) s = fmaf(raw[c], raw[c], s);
+  const float rq = 1.f / sqrtf(block_sum_256(s, red) / (float)a.q_rank + a.eps);
+  T* cq = (T*)a.cq + (size_t)t * a.q_rank;
+  for (int c = tid; c < a.q_rank; c += 256) El<T>::st(cq + c, raw[c] * rq * a.qn_w[c]);
+  const int64_t slot = a.slots[t];
+  if (slot < 0) return;
+  const float* kv = raw + a.q_rank;
+  s = 0.f;
+  for (int c = tid; c < a.kv_rank; c += 256) s = fmaf(kv[c], kv[c], s);
+  const float rk = 1.f / sqrtf(block_sum_256(s, red) / (float)a.kv_rank + a.eps);
+  T* row = (T*)a.cache + slot * a.cache_ld;
+  for (int c = tid; c < a.kv_rank; c += 256) El<T>::st(row + c, kv[c] * rk * a.kvn_w[c]);
+  const float p = (float)a.positions[t];
+  const float* r = kv + a.kv_rank;
+  for (int i = tid; i < a.rot_dim / 2 + (a.rot_dim & 1); i += 256) {
+    if (i < a.rot.pairs) {
+      float c, sn;
+      rot_cos_sin(a.rot, i, p, &c, &sn);
+      const float u = r[2 * i], v = r[2 * i + 1];
+      El<T>::st(row + a.kv_rank + 2 * i, u * c - v * sn);
+      El<T>::st(row + a.kv_rank + 2 * i + 1, v * c + u * sn);
+    } else {
+      El<T>::st(row + a.kv_rank + 2 * i, r[2 * i]);
+      if (2 * i + 1 < a.rot_dim) El<T>::st(row + a.kv_rank + 2 * i + 1, r[2 * i + 1]);
+    }
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void stk_rope_heads_kernel(const T* in, int in_ld, int in_hs, int in_off, T* out, int out_ld, int out_hs, int out_off,
+                                                             int n, int H, const int64_t* positions, StkRotary rot) {
+  const int t = blockIdx.x;
+  const float p = (float)positions[t];
+  const int half = n / 2 + (n & 1);
+  for (int e = threadIdx.x; e < H * half; e += 256) {
+    const int h = e / half, i = e % half;
+    const T* src = in + (size_t)t * in_ld + h * in_hs + in_off;
+    T* dst = out + (size_t)t * out_ld + h * out_hs + out_off;
+    if (i < rot.pairs) {
+      float c, sn;
+      rot_cos_sin(rot, i, p, &c, &sn);
+      const float u = El<T>::ld(src + 2 * i), v = El<T>::ld(src + 2 * i + 1);
+      El<T>::st(dst + 2 * i, u * c - v * sn);
+      El<T>::st(dst + 2 * i + 1, v * c + u * sn);
+    } else {
+      El<T>::st(dst + 2 * i, El<T>::ld(src + 2 * i));
+      if (2 * i + 1 < n) El<T>::st(dst + 2 * i + 1, El<T>::ld(src + 2 * i + 1));
+    }
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ whole-projection q / k norm + cache rows
+template <typename T>
+__global__ __launch_bounds__(256) void stk_qk_norm_store_kernel(const float* raw, int ld, int nq, int nk, int nv, const float* q_w, const float* k_w,
+                                                                float eps, T* q_out, T* kc, T* vc, const int64_t* slots) {
+  __shared__ float red[4];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const float* r = raw + (size_t)t * ld;
+  float rq = 1.f, rk = 1.f;
+  if (q_w) {
+    float s = 0.f;
+    for (int c = tid; c < nq; c += 256) s = fmaf(r[c], r[c], s);
+    rq = 1.f / sqrtf(block_sum_256(s, red) / (float)nq + eps);
+  }
+  for (int c = tid; c < nq; c += 256) El<T>::st(q_out + (size_t)t * nq + c, q_w ? r[c] * rq * q_w[c] : r[c]);
+  const int64_t slot = slots[t];
+  if (slot < 0) return;
+  if (k_w) {
+    float s = 0.f;
+    for (int c = tid; c < nk; c += 256) s = fmaf(r[nq + c], r[nq + c], s);
+    rk = 1.f / sqrtf(block_sum_256(s, red) / (float)nk + eps);
+  }
+  for (int c = tid; c < nk; c += 256) El<T>::st(kc + slot * nk + c, k_w ? r[nq + c] * rk * k_w[c] : r[nq + c]);
+  for (int c = tid; c < nv; c += 256) El<T>::st(vc + slot * nv + c, r[nq + nk + c]);
+}
+
+// ------------------------------------------------------------------------------------------------ attention without softmax
+// A workgroup owns QT query rows of one sequence and ALL heads (the mixing of the heads' weights needs every head's weight of a (query,
+// key) pair in one place).  Key tiles of KT tokens, aligned to absolute positions; tiles that no row can see (between the kept first
+// tokens and the window) are skipped.  Per tile: scores and weights head by head into LDS, the mix, then the value product with the
+// accumulators in registers: thread = (row, every TPR-th output channel).
+template <typename T, int QT, int NACC>
+__global__ __launch_bounds__(256) void stk_sig_attn_kernel(StkSigAttnArgs a, int KT) {
+  extern __shared__ float lds[];
+  constexpr int TPR = 256 / QT;
+  const int dim = a.dim, vdim = a.vdim, H = a.H, G = a.G, HG = H / G, kld = dim + 1, GV = G * vdim, HV = H * vdim;
+  float* qs = lds;                       // [QT][dim]
+  float* ks = qs + QT * dim;             // [KT][dim + 1]
+  float* ws = ks + KT * kld;             // [H][QT][KT]
+  float* ms = ws + H * QT * KT;          // [H][QT][KT] (mixed; aliases ws without a mixing matrix)
+  float* vs = a.talk ? ms + H * QT * KT : ms;  // [KT][G * vdim]
+  float* tk = vs + KT * GV;              // [H][H]
+  if (!a.talk) ms = ws;
+  const int b = blockIdx.y, tid = threadIdx.x;
+  const int q0 = a.cu_q ? a.cu_q[b] : b, q1 = a.cu_q ? a.cu_q[b + 1] : b + 1;
+  const int t0 = q0 + blockIdx.x * QT;
+  if (t0 >= q1) return;
+  const int nq = min(QT, q1 - t0);
+  int64_t pmin = a.positions[t0], pmax = pmin;
+  for (int r = 1; r < nq; r++) pmin = min(pmin, a.positions[t0 + r]), pmax = max(pmax, a.positions[t0 + r]);
+  const int n_keys = (int)min((int64_t)a.context_lens[b], pmax + 1);
+  if (a.talk)
+    for (int i = tid; i < H * H; i += 256) tk[i] = a.talk[i];
+  const T* q = (const T*)a.q;
+  const T* kc = (const T*)a.kc;
+  const T* vc = (const T*)a.vc;
+  const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
+  float acc[NACC];
+#pragma unroll
+  for (int i = 0; i < NACC; i++) acc[i] = 0.f;
+  const int pr = tid / TPR, pl = tid % TPR;  // value phase: row, first channel
+  const int win_first = a.window > 0 ? (int)(max((int64_t)0, pmin - a.window + 1) / KT) * KT : 0;
+  const int keep_end = a.window > 0 ? (max(a.keep_first, 0) + KT - 1) / KT * KT : 0;
+  for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
+    if (a.window > 0 && kt0 >= keep_end && kt0 < win_first) {  // nothing between the kept tokens and the window is seen
+      kt0 = win_first - KT;
+      continue;
+    }
+    for (int g = 0; g < G; g++) {
+      __syncthreads();
+      for (int i = tid; i < KT * dim; i += 256) {
+        const int j = i / dim, d = i % dim, key = kt0 + j;
+        float v = 0.f;
+        if (key < n_keys) {
+          const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
+          v = El<T>::ld(kc + slot * (G * dim) + g * dim + d);
+        }
+        ks[j * kld + d] = v;
+      }
+      for (int hh = 0; hh < HG; hh++) {
+        const int h = g * HG + hh;
+        __syncthreads();
+        for (int i = tid; i < QT * dim; i += 256) {
+          const int r = i / dim, d = i % dim;
+          qs[i] = r < nq ? El<T>::ld(q + (size_t)(t0 + r) * a.ldq + h * dim + d) : 0.f;
+        }
+        __syncthreads();
+        const float slope = a.slopes ? a.slopes[h] : 0.f, hb = a.head_bias ? a.head_bias[h] : 0.f;
+        for (int i = tid; i < QT * KT; i += 256) {
+          const int r = i / KT, j = i % KT, key = kt0 + j;
+          float w = 0.f;
+          if (r < nq && key < n_keys) {
+            const int64_t p = a.positions[t0 + r];
+            if (key <= p && (a.window <= 0 || p - key < a.window || key < a.keep_first)) {
+              float d0 = 0.f;
+              for (int d = 0; d < dim; d++) d0 = fmaf(qs[r * dim + d], ks[j * kld + d], d0);
+              w = sigmoidf_(d0 * a.scale - slope * (float)(p - key) + hb);
+            }
+          }
+          ws[(h * QT + r) * KT + j] = w;
+        }
+      }
+    }
+    __syncthreads();
+    if (a.talk) {
+      for (int i = tid; i < QT * KT; i += 256) {
+        const int r = i / KT, j = i % KT;
+        for (int h = 0; h < H; h++) {
+          float s = 0.f;
+          for (int g2 = 0; g2 < H; g2++) s = fmaf(tk[h * H + g2], ws[(g2 * QT + r) * KT + j], s);
+          ms[(h * QT + r) * KT + j] = s;
+        }
+      }
+    }
+    for (int i = tid; i < KT * GV; i += 256) {
+      const int j = i / GV, c = i % GV, key = kt0 + j;
+      float v = 0.f;
+      if (key < n_keys) {
+        const int64_t slot = (int64_t)bt[key / a.BS] * a.BS + key % a.BS;
+        v = El<T>::ld(vc + slot * GV + c);
+      }
+      vs[i] = v;
+    }
+    __syncthreads();
+    const int nj = min(KT, n_keys - kt0);
+#pragma unroll
+    for (int n = 0; n < NACC; n++) {
+      const int c = pl + n * TPR;
+      if (c < HV) {
+        const int h = c / vdim, d = c % vdim, g = h / HG;
+        const float* mw = ms + (h * QT + pr) * KT;
+        const float* vv = vs + g * vdim + d;
+        float o = acc[n];
+        for (int j = 0; j < nj; j++) o = fmaf(mw[j], vv[j * GV], o);
+        acc[n] = o;
+      }
+    }
+  }
+  if (pr >= nq) return;
+  T* out = (T*)a.out + (size_t)(t0 + pr) * HV;
+#pragma unroll
+  for (int n = 0; n < NACC; n++) {
+    const int c = pl + n * TPR;
+    if (c < HV) {
+      float o = acc[n];
+      if (a.gate) o *= sigmoidf_(a.gate[(size_t)(t0 + pr) * a.gate_ld + c]);
+      El<T>::st(out + c, o);
+    }
+  }
+}
+
+}  // namespace
+
+// ================================================================================================ launchers
+void vra_stack_dyt(float* x, const float* add, const float* w, const float* b, float alpha, void* h, int T, int W, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(x && w && b && h && T > 0 && W > 0, "stack dyt: null pointer or empty shape");
+  const int64_t n = (int64_t)T * W;
+  const int grid = (int)std::min<int64_t>((n + 255) / 256, 4096);
+  if (dtype == VRA_F32) launch_checked("stack dyt", [&] { stk_dyt_kernel<float><<<grid, 256, 0, as_stream(stream)>>>(x, add, w, b, alpha, (float*)h, W, n); });
+  else launch_checked("stack dyt", [&] { stk_dyt_kernel<uint16_t><<<grid, 256, 0, as_stream(stream)>>>(x, add, w, b, alpha, (uint16_t*)h, W, n); });
+}
+
+void vra_stack_latent_prep(const StkLatentPrepArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.raw && a.qn_w && a.kvn_w && a.cq && a.cache && a.slots && a.positions && a.T > 0, "stack latent prep: null pointer or empty shape");
+  VRA_CHECK_ARG(a.q_rank > 0 && a.kv_rank > 0 && a.rot_dim >= 0 && a.ld >= a.q_rank + a.kv_rank + a.rot_dim && a.cache_ld >= a.kv_rank + a.rot_dim,
+                "stack latent prep: row shorter than its parts");
+  VRA_CHECK_ARG(a.rot.pairs * 2 <= a.rot_dim && (a.rot.pairs == 0 || a.rot.freq_hi), "stack latent prep: more rotated pairs than the rotated part holds");
+  if (dtype == VRA_F32) launch_checked("stack latent prep", [&] { stk_latent_prep_kernel<float><<<a.T, 256, 0, as_stream(stream)>>>(a); });
+  else launch_checked("stack latent prep", [&] { stk_latent_prep_kernel<uint16_t><<<a.T, 256, 0, as_stream(stream)>>>(a); });
+}
+
+void vra_stack_rope_heads(const void* in, int in_ld, int in_hs, int in_off, void* out, int out_ld, int out_hs, int out_off, int n, int H,
+                          const int64_t* positions, const StkRotary& rot, int T, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(in && out && positions && T > 0 && H > 0 && n > 0, "stack rope: null pointer or empty shape");
+  VRA_CHECK_ARG(rot.pairs * 2 <= n && (rot.pairs == 0 || rot.freq_hi), "stack rope: more rotated pairs than the vector holds");
+  if (dtype == VRA_F32)
+    launch_checked("stack rope", [&] {
+      stk_rope_heads_kernel<float><<<T, 256, 0, as_stream(stream)>>>((const float*)in, in_ld, in_hs, in_off, (float*)out, out_ld, out_hs, out_off, n, H, positions, rot);
+    });
+  else
+    launch_checked("stack rope", [&] {
+      stk_rope_heads_kernel<uint16_t><<<T, 256, 0, as_stream(stream)>>>((const uint16_t*)in, in_ld, in_hs, in_off, (uint16_t*)out, out_ld, out_hs, out_off, n, H,
+                                                                        positions, rot);
+    });
+}
+
+void vra_stack_qk_norm_store(const float* raw, int ld, int nq, int nk, int nv, const float* q_w, const float* k_w, float eps, void* q_out, void* kc,
+                             void* vc, const int64_t* slots, int T, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(raw && q_out && kc && vc && slots && T > 0 && nq > 0 && nk > 0 && nv > 0 && ld >= nq + nk + nv, "stack qk norm: null pointer or empty shape");
+  if (dtype == VRA_F32)
+    launch_checked("stack qk norm", [&] {
+      stk_qk_norm_store_kernel<float><<<T, 256, 0, as_stream(stream)>>>(raw, ld, nq, nk, nv, q_w, k_w, eps, (float*)q_out, (float*)kc, (float*)vc, slots);
+    });
+  else
+    launch_checked("stack qk norm", [&] {
+      stk_qk_norm_store_kernel<uint16_t><<<T, 256, 0, as_stream(stream)>>>(raw, ld, nq, nk, nv, q_w, k_w, eps, (uint16_t*)q_out, (uint16_t*)kc, (uint16_t*)vc, slots);
+    });
+}
+
+void vra_stack_sigmoid_attention(const StkSigAttnArgs& a, int dtype, int64_t stream) {
+  VRA_CHECK_ARG(a.q && a.out && a.kc && a.vc && a.positions && a.block_tables && a.context_lens, "stack sigmoid attention: null pointer");
+  VRA_CHECK_ARG(a.B > 0 && a.H > 0 && a.G > 0 && a.H % a.G == 0 && a.dim > 0 && a.vdim > 0 && a.BS > 0 && a.max_blocks > 0 && a.max_q > 0,
+                "stack sigmoid attention: heads must be a multiple of kv heads, sizes positive");
+  VRA_CHECK_ARG(!a.gate || a.gate_ld >= a.H * a.vdim, "stack sigmoid attention: gate rows shorter than the output");
+  hipStream_t st = as_stream(stream);
+  const int HV = a.H * a.vdim;
+  const bool decode = !a.cu_q;
+  int qt, nacc;
+  if (decode) qt = 1, nacc = HV <= 4096 ? 16 : 64;
+  else if (HV <= 256) qt = 16, nacc = 16;
+  else if (HV <= 1024) qt = 16, nacc = 64;
+  else if (HV <= 4096) qt = 4, nacc = 64;
+  else qt = 1, nacc = 64;
+  VRA_CHECK_ARG(HV <= (256 / qt) * nacc, "stack sigmoid attention: more output channels than the kernel's accumulators hold");
+  auto need = [&](int kt) {
+    return ((size_t)qt * a.dim + (size_t)kt * (a.dim + 1) + (size_t)(a.talk ? 2 : 1) * a.H * qt * kt + (size_t)kt * a.G * a.vdim + (size_t)a.H * a.H) * sizeof(float);
+  };
+  int kt = 64;
+  while (kt > 8 && need(kt) > 64 * 1024) kt >>= 1;
+  VRA_CHECK_ARG(need(kt) <= 64 * 1024, "stack sigmoid attention: heads do not fit LDS");
+  const size_t lds = need(kt);
+  dim3 grid(decode ? 1 : (a.max_q + qt - 1) / qt, a.B);
+#define STK_SG(TT, QTV, NA) launch_checked("stack sigmoid attention", [&] { stk_sig_attn_kernel<TT, QTV, NA><<<grid, 256, lds, st>>>(a, kt); })
+#define STK_SG_T(TT)                          \
+  if (qt == 16 && nacc == 16) STK_SG(TT, 16, 16); \
+  else if (qt == 16) STK_SG(TT, 16, 64);          \
+  else if (qt == 4) STK_SG(TT, 4, 64);            \
+  else if (nacc == 16) STK_SG(TT, 1, 16);         \
+  else STK_SG(TT, 1, 64)
+  if (dtype == VRA_F32) {
+    STK_SG_T(float);
+  } else {
+    STK_SG_T(uint16_t);
+  }
+#undef STK_SG_T
+#undef STK_SG
+}
+
+// ================================================================================================ C entry points (one operator each)
+extern "C" void vra_stack_op_dyt(float* x, const float* add, const float* w, const float* b, float alpha, void* h, int32_t T, int32_t W, int32_t dtype,
+                                 int64_t stream) {
+  vra_stack_dyt(x, add, w, b, alpha, h, T, W, dtype, stream);
+}
+extern "C" void vra_stack_op_latent_prep(const float* raw, int32_t ld, int32_t q_rank, int32_t kv_rank, int32_t rot_dim, const float* qn_w,
+                                         const float* kvn_w, float eps, void* cq, void* cache, int32_t cache_ld, const int64_t* slots,
+                                         const int64_t* positions, const float* freq_hi, const float* freq_lo, int32_t pairs, float mag, int32_t T,
+                                         int32_t dtype, int64_t stream) {
+  StkLatentPrepArgs a;
+  a.raw = raw, a.ld = ld, a.q_rank = q_rank, a.kv_rank = kv_rank, a.rot_dim = rot_dim, a.qn_w = qn_w, a.kvn_w = kvn_w, a.eps = eps, a.cq = cq;
+  a.cache = cache, a.cache_ld = cache_ld, a.slots = slots, a.positions = positions, a.T = T;
+  a.rot.freq_hi = freq_hi, a.rot.freq_lo = freq_lo, a.rot.pairs = pairs, a.rot.mag = mag;
+  vra_stack_latent_prep(a, dtype, stream);
+}
+extern "C" void vra_stack_op_rope_heads(const void* in, int32_t in_ld, int32_t in_hs, int32_t in_off, void* out, int32_t out_ld, int32_t out_hs,
+                                        int32_t out_off, int32_t n, int32_t H, const int64_t* positions, const float* freq_hi, const float* freq_lo,
+                                        int32_t pairs, float mag, int32_t T, int32_t dtype, int64_t stream) {
+  StkRotary r;
+  r.freq_hi = freq_hi, r.freq_lo = freq_lo, r.pairs = pairs, r.mag = mag;
+  vra_stack_rope_heads(in, in_ld, in_hs, in_off, out, out_ld, out_hs, out_off, n, H, positions, r, T, dtype, stream);
+}
+extern "C" void vra_stack_op_qk_norm_store(const float* raw, int32_t ld, int32_t nq, int32_t nk, int32_t nv, const float* q_w, const float* k_w, float eps,
+                                           void* q_out, void* kc, void* vc, const int64_t* slots, int32_t T, int32_t dtype, int64_t stream) {
+  vra_stack_qk_norm_store(raw, ld, nq, nk, nv, q_w, k_w, eps, q_out, kc, vc, slots, T, dtype, stream);
+}
+extern "C" void vra_stack_op_sigmoid_attention(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                               const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                                               int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks, float scale,
+                                               int32_t window, int32_t keep_first, const float* slopes, const float* head_bias, const float* talk,
+                                               const float* gate, int32_t gate_ld, int32_t dtype, int64_t stream) {
+  StkSigAttnArgs a;
+  a.q = q, a.ldq = ldq, a.out = out, a.kc = kc, a.vc = vc, a.positions = positions, a.block_tables = block_tables, a.context_lens = context_lens;
+  a.cu_q = cu_q, a.B = B, a.T = T, a.max_q = max_q, a.H = H, a.G = G, a.dim = dim, a.vdim = vdim, a.BS = BS, a.max_blocks = max_blocks;
+  a.scale = scale, a.window = window, a.keep_first = keep_first, a.slopes = slopes, a.head_bias = head_bias, a.talk = talk, a.gate = gate;
+  a.gate_ld = gate_ld;
+  vra_stack_sigmoid_attention(a, dtype, stream);
+}
+// the matrix product with every option of StkGemmArgs: bias, batched form, kind of the gated pair
+extern "C" void vra_stack_op_gemm_ex(const void* a, int32_t lda, const void* w, void* out, int32_t ldo, int32_t out_f32, int32_t M, int32_t N, int32_t K,
+                                     float alpha, const float* bias, int32_t epi, int32_t act, int32_t batch, int64_t a_batch_stride,
+                                     int64_t w_batch_stride, int64_t out_batch_stride, int32_t dtype, int64_t stream) {
+  StkGemmArgs g;
+  g.a = a, g.lda = lda, g.w = w, g.out = out, g.ldo = ldo, g.out_f32 = out_f32, g.M = M, g.N = N, g.K = K, g.alpha = alpha, g.bias = bias;
+  g.epi = epi, g.act = act, g.batch = batch, g.a_batch_stride = a_batch_stride, g.w_batch_stride = w_batch_stride, g.out_batch_stride = out_batch_stride;
+  vra_stack_gemm(g, dtype, stream);
+}
+// the softmax attention with a sink and a latent cache's row layout
+extern "C" void vra_stack_op_attention_ex(const void* q, int32_t ldq, void* out, const void* kc, const void* vc, const int64_t* positions,
+                                          const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
+                                          int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks, float scale,
+                                          const float* sink, int32_t k_ld, int32_t v_ld, int32_t dtype, int64_t stream) {
+  StkAttnArgs a;
+  a.q = q, a.ldq = ldq, a.out = out, a.kc = kc, a.vc = vc, a.positions = positions, a.block_tables = block_tables, a.context_lens = context_lens;
+  a.cu_q = cu_q, a.B = B, a.T = T, a.max_q = max_q, a.H = H, a.G = G, a.dim = dim, a.vdim = vdim, a.BS = BS, a.max_blocks = max_blocks;
+  a.scale = scale, a.sink = sink, a.k_ld = k_ld, a.v_ld = v_ld;
+  vra_stack_attention(a, dtype, stream);
+}

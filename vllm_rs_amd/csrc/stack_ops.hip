@@ -7,36 +7,15 @@
 // of a step, on a row's place in the batch or on the pages it uses — so a token's result does not depend on how its prompt was cut.
 #include <math.h>
 
-#include "common.cuh"
+#include "stack_common.cuh"
 #include "stack_launch.h"
 
 namespace {
 
-template <typename T>
-struct El;
-template <>
-struct El<float> {
-  static __device__ __forceinline__ float ld(const float* p) { return *p; }
-  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
-  static __device__ __forceinline__ float rnd(float v) { return v; }
-};
-template <>
-struct El<uint16_t> {
-  static __device__ __forceinline__ float ld(const uint16_t* p) { return BF16::to_f32(*p); }
-  static __device__ __forceinline__ void st(uint16_t* p, float v) { *p = BF16::from_f32(v); }
-  static __device__ __forceinline__ float rnd(float v) { return BF16::to_f32(BF16::from_f32(v)); }
-};
-
-__device__ __forceinline__ float wave_sum(float v) {
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
-}
-__device__ __forceinline__ float sigmoidf_(float z) { return 1.f / (1.f + expf(-z)); }
-__device__ __forceinline__ float gated_pair(float g, float u, float limit, float act_alpha) {
+__device__ __forceinline__ float gelu_tanh_(float z) { return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+// act 0: min(g, L) * sigmoid(act_alpha * min(g, L)) * (clamp(u, +-L) + 1);  act 1: gelu_tanh(g) * u
+__device__ __forceinline__ float gated_pair(float g, float u, float limit, float act_alpha, int act = 0) {
+  if (act == 1) return gelu_tanh_(g) * u;
   if (limit > 0.f) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
@@ -53,8 +32,11 @@ __global__ __launch_bounds__(256) void stk_embed_sinpos_kernel(const uint32_t* i
   if (id >= (uint32_t)V) id = 0;
   const float p = (float)pos[t];
   for (int c = threadIdx.x; c < W; c += 256) {
-    const float ang = p * inv_freq[c >> 1];
-    const float pe = (c & 1) ? cosf(ang) : sinf(ang);
+    float pe = 0.f;
+    if (inv_freq) {
+      const float ang = p * inv_freq[c >> 1];
+      pe = (c & 1) ? cosf(ang) : sinf(ang);
+    }
     x[(size_t)t * W + c] = El<T>::ld(embed + (size_t)id * W + c) + pe;
   }
 }
@@ -177,8 +159,9 @@ __global__ __launch_bounds__(256) void stk_gemm_simple_kernel(StkGemmArgs g) {
     group = g.tile_group[blockIdx.x];
     if (group < 0) return;
   }
-  const T* A = (const T*)g.a;
-  const T* Wt = (const T*)g.w + (int64_t)group * g.w_group_stride;
+  const T* A = (const T*)g.a + (int64_t)blockIdx.z * g.a_batch_stride;
+  const T* Wt = (const T*)g.w + (int64_t)group * g.w_group_stride + (int64_t)blockIdx.z * g.w_batch_stride;
+  const int64_t ob = (int64_t)blockIdx.z * g.out_batch_stride;
   if (tid < TM) {
     const int r = m0 + tid;
     int idx = r < g.M ? (g.a_row ? g.a_row[r] : r) : -1;
@@ -222,9 +205,9 @@ __global__ __launch_bounds__(256) void stk_gemm_simple_kernel(StkGemmArgs g) {
     for (int j = 0; j < 4; j++) {
       const int n = n0 + tx * 4 + j;
       if (n >= g.N) continue;
-      const float v = acc[i][j] * g.alpha;
-      if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = v;
-      else El<T>::st((T*)g.out + (int64_t)orow * g.ldo + n, v);
+      const float v = acc[i][j] * g.alpha + (g.bias ? g.bias[n] : 0.f);
+      if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = v;
+      else El<T>::st((T*)g.out + ob + (int64_t)orow * g.ldo + n, v);
     }
   }
 }
@@ -242,8 +225,9 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
     group = g.tile_group[blockIdx.x];
     if (group < 0) return;
   }
-  const uint16_t* A = (const uint16_t*)g.a;
-  const uint16_t* Wt = (const uint16_t*)g.w + (int64_t)group * g.w_group_stride;
+  const uint16_t* A = (const uint16_t*)g.a + (int64_t)blockIdx.z * g.a_batch_stride;
+  const uint16_t* Wt = (const uint16_t*)g.w + (int64_t)group * g.w_group_stride + (int64_t)blockIdx.z * g.w_batch_stride;
+  const int64_t ob = (int64_t)blockIdx.z * g.out_batch_stride;
   const int m_base = blockIdx.x * (16 * MT * WM) + wm * 16 * MT;
   const int n_base = blockIdx.y * (16 * NT * WN) + wn * 16 * NT;
   const uint16_t* ap[MT];
@@ -320,9 +304,9 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
         for (int j = 0; j < 4; j++) {
           const int n = (n_base + nt * 16) / 2 + oct * 4 + j;
           if (n >= g.N / 2) continue;
-          const float y = gated_pair(acc[mt][nt][j], acc[mt][nt + 1][j], g.limit, g.act_alpha);
-          if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = y;
-          else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(y);
+          const float y = gated_pair(acc[mt][nt][j], acc[mt][nt + 1][j], g.limit, g.act_alpha, g.act);
+          if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = y;
+          else ((uint16_t*)g.out)[ob + (int64_t)orow * g.ldo + n] = BF16::from_f32(y);
         }
     } else {
 #pragma unroll
@@ -330,9 +314,9 @@ __global__ __launch_bounds__(64 * WM * WN) void stk_gemm_mfma_kernel(StkGemmArgs
         for (int j = 0; j < 4; j++) {
           const int n = n_base + nt * 16 + oct * 4 + j;
           if (n >= g.N) continue;
-          const float v = acc[mt][nt][j] * g.alpha;
-          if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = v;
-          else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(v);
+          const float v = acc[mt][nt][j] * g.alpha + (g.bias ? g.bias[n] : 0.f);
+          if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = v;
+          else ((uint16_t*)g.out)[ob + (int64_t)orow * g.ldo + n] = BF16::from_f32(v);
         }
     }
   }
@@ -350,8 +334,9 @@ __global__ __launch_bounds__(512) void stk_gemm_mfma_small_kernel(StkGemmArgs g)
     group = g.tile_group[blockIdx.x];
     if (group < 0) return;
   }
-  const uint16_t* A = (const uint16_t*)g.a;
-  const uint16_t* Wt = (const uint16_t*)g.w + (int64_t)group * g.w_group_stride;
+  const uint16_t* A = (const uint16_t*)g.a + (int64_t)blockIdx.z * g.a_batch_stride;
+  const uint16_t* Wt = (const uint16_t*)g.w + (int64_t)group * g.w_group_stride + (int64_t)blockIdx.z * g.w_batch_stride;
+  const int64_t ob = (int64_t)blockIdx.z * g.out_batch_stride;
   const int m_base = blockIdx.x * 16, n_base = blockIdx.y * 32;
   const int r = m_base + rq;
   const int idx = r < g.M ? (g.a_row ? g.a_row[r] : r) : -1;
@@ -409,27 +394,27 @@ __global__ __launch_bounds__(512) void stk_gemm_mfma_small_kernel(StkGemmArgs g)
     if (c >= 16) return;
     const int n = n_base / 2 + c;
     if (n >= g.N / 2) return;
-    const float y = gated_pair(total(c), total(16 + c), g.limit, g.act_alpha);
-    if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = y;
-    else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(y);
+    const float y = gated_pair(total(c), total(16 + c), g.limit, g.act_alpha, g.act);
+    if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = y;
+    else ((uint16_t*)g.out)[ob + (int64_t)orow * g.ldo + n] = BF16::from_f32(y);
   } else {
     const int n = n_base + c;
     if (n >= g.N) return;
-    const float v = total(c) * g.alpha;
-    if (g.out_f32) ((float*)g.out)[(int64_t)orow * g.ldo + n] = v;
-    else ((uint16_t*)g.out)[(int64_t)orow * g.ldo + n] = BF16::from_f32(v);
+    const float v = total(c) * g.alpha + (g.bias ? g.bias[n] : 0.f);
+    if (g.out_f32) ((float*)g.out)[ob + (int64_t)orow * g.ldo + n] = v;
+    else ((uint16_t*)g.out)[ob + (int64_t)orow * g.ldo + n] = BF16::from_f32(v);
   }
 }
 
 // ------------------------------------------------------------------------------------------------ activations
 template <typename T>
-__global__ __launch_bounds__(256) void stk_gated_act_kernel(const float* gu, T* out, int F, float limit, float act_alpha) {
+__global__ __launch_bounds__(256) void stk_gated_act_kernel(const float* gu, T* out, int F, float limit, float act_alpha, int act) {
   const int m = blockIdx.x;
   const int Fp = (F + 15) / 16 * 16;
   for (int f = threadIdx.x; f < F; f += 256) {
     const int b = f >> 4, i = f & 15;
     const float gv = gu[(size_t)m * 2 * Fp + (2 * b) * 16 + i], uv = gu[(size_t)m * 2 * Fp + (2 * b + 1) * 16 + i];
-    El<T>::st(out + (size_t)m * Fp + f, gated_pair(gv, uv, limit, act_alpha));
+    El<T>::st(out + (size_t)m * Fp + f, gated_pair(gv, uv, limit, act_alpha, act));
   }
   for (int f = F + threadIdx.x; f < Fp; f += 256) El<T>::st(out + (size_t)m * Fp + f, 0.f);
 }
@@ -557,12 +542,13 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_kernel(StkAttnArgs a) {
   float m[4], l[4], acc[4][4];
   for (int i = 0; i < 4; i++) {
     m[i] = -INFINITY, l[i] = 0.f;
+    if (a.sink) m[i] = a.sink[h], l[i] = 1.f;  // the sink: one more term exp(sink - m) of the denominator, present from the start
     for (int r = 0; r < 4; r++) acc[i][r] = 0.f;
   }
   const T* kc = (const T*)a.kc;
   const T* vc = (const T*)a.vc;
   const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
-  const int kdim = a.G * dim, vd_all = a.G * vdim;
+  const int kdim = a.k_ld ? a.k_ld : a.G * dim, vd_all = a.v_ld ? a.v_ld : a.G * vdim;
   for (int kt0 = 0; kt0 < n_keys; kt0 += KT) {
     __syncthreads();
     for (int i = tid; i < KT * dim; i += 256) {
@@ -671,10 +657,11 @@ __global__ __launch_bounds__(256) void stk_attn_prefill_mfma_kernel(StkAttnArgs 
   const uint16_t* kc = (const uint16_t*)a.kc;
   const uint16_t* vc = (const uint16_t*)a.vc;
   const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
-  const int kdim = a.G * dim, vd_all = a.G * vdim;
+  const int kdim = a.k_ld ? a.k_ld : a.G * dim, vd_all = a.v_ld ? a.v_ld : a.G * vdim;
   f32x4 acc[VT];
   for (int t = 0; t < VT; t++) acc[t] = vra_zero_acc();
   float m = -INFINITY, l = 0.f;
+  if (a.sink) m = a.sink[h], l = oct == 0 ? 1.f : 0.f;  // (the four lanes of a row add their sums at the end: the sink counts once)
   const bool capped = a.softcap > 0.f;
   const float two_inv_cap = capped ? 2.f / a.softcap : 0.f, two_cap = 2.f * a.softcap;
   const int key_end = (int)min((int64_t)n_keys, pq + 1);  // this row sees the keys below key_end
@@ -860,10 +847,11 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
   const T* kc = (const T*)a.kc;
   const T* vc = (const T*)a.vc;
   const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
-  const int kdim = a.G * dim, vd_all = a.G * vdim;
+  const int kdim = a.k_ld ? a.k_ld : a.G * dim, vd_all = a.v_ld ? a.v_ld : a.G * vdim;
   float m = -INFINITY, l = 0.f, acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (a.sink && wave == 0) m = a.sink[h], l = 1.f;
   // 16-bit values in whole octets: the value phase reads 16 bytes a lane (oc = channel octets rounded up to a power of two)
-  const bool vec = sizeof(T) == 2 && vdim % 8 == 0 && ((uintptr_t)vc % 16) == 0;
+  const bool vec = sizeof(T) == 2 && vdim % 8 == 0 && vd_all % 8 == 0 && ((uintptr_t)vc % 16) == 0;
   int oc = 1;
   while (oc * 8 < vdim) oc <<= 1;
   const int co = lane & (oc - 1), kg = lane / oc, kpar = 64 / oc;
@@ -947,13 +935,6 @@ __global__ __launch_bounds__(64 * STK_DW) void stk_attn_decode_kernel(StkAttnArg
   }
 }
 
-template <typename F>
-void launch_checked(const char* what, F f) {
-  f();
-  const hipError_t e = hipGetLastError();
-  if (e != hipSuccess) vra_set_error("%s: %s", what, hipGetErrorString(e));
-}
-
 }  // namespace
 
 // ================================================================================================ launchers
@@ -963,33 +944,35 @@ void vra_stack_gemm(const StkGemmArgs& g, int dtype, int64_t stream) {
   VRA_CHECK_ARG(g.a && g.w && g.out && g.M > 0 && g.N > 0 && g.K > 0, "stack gemm: null pointer or empty shape");
   VRA_CHECK_ARG(dtype == VRA_BF16 || dtype == VRA_F32, "stack gemm: dtype must be bf16 or f32");
   VRA_CHECK_ARG(!g.tile_group || g.granule == 16 || g.granule == 64, "stack gemm: granule must be 16 or 64");
+  VRA_CHECK_ARG(g.batch >= 1 && (g.batch == 1 || !g.tile_group), "stack gemm: a batched product has no row groups");
   hipStream_t st = as_stream(stream);
+  const int nb = g.batch;
   const bool big = g.tile_group ? g.granule == 64 : g.M > 32;
   const bool mfma = dtype == VRA_BF16 && g.K % 8 == 0 && g.lda % 8 == 0 && ((uintptr_t)g.a % 16 == 0) && ((uintptr_t)g.w % 16 == 0) &&
-                    (g.w_group_stride % 8 == 0);
+                    (g.w_group_stride % 8 == 0) && (g.a_batch_stride % 8 == 0) && (g.w_batch_stride % 8 == 0);
   VRA_CHECK_ARG(g.epi == 0 || (mfma && g.N % 32 == 0), "stack gemm: the gated epilogue needs the bf16 MFMA path and whole gate / up blocks");
   if (mfma) {
-    if (big && !g.tile_group && !g.a_scale && g.M >= 256 && (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) >= 256) {
+    if (big && !g.tile_group && !g.a_scale && g.M >= 256 && (int64_t)((g.M + 127) / 128) * ((g.N + 127) / 128) * nb >= 256) {
       // enough 128 x 128 tiles to fill the chip: a wave owns 64 x 64 (16 MFMAs per 8 fragment requests instead of 8 per 6)
-      dim3 grid((g.M + 127) / 128, (g.N + 127) / 128);
+      dim3 grid((g.M + 127) / 128, (g.N + 127) / 128, nb);
       launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<4, 4, 2, 2, false><<<grid, 256, 0, st>>>(g); });
     } else if (big) {
-      dim3 grid((g.M + 63) / 64, (g.N + 127) / 128);
+      dim3 grid((g.M + 63) / 64, (g.N + 127) / 128, nb);
       if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, true><<<grid, 256, 0, st>>>(g); });
       else launch_checked("stack gemm", [&] { stk_gemm_mfma_kernel<2, 4, 2, 2, false><<<grid, 256, 0, st>>>(g); });
     } else {
-      dim3 grid((g.M + 15) / 16, (g.N + 31) / 32);
+      dim3 grid((g.M + 15) / 16, (g.N + 31) / 32, nb);
       if (g.a_scale) launch_checked("stack gemm", [&] { stk_gemm_mfma_small_kernel<true><<<grid, 512, 0, st>>>(g); });
       else launch_checked("stack gemm", [&] { stk_gemm_mfma_small_kernel<false><<<grid, 512, 0, st>>>(g); });
     }
     return;
   }
   if (big) {
-    dim3 grid((g.M + 63) / 64, (g.N + 63) / 64);
+    dim3 grid((g.M + 63) / 64, (g.N + 63) / 64, nb);
     if (dtype == VRA_F32) launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<float, 4><<<grid, 256, 0, st>>>(g); });
     else launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<uint16_t, 4><<<grid, 256, 0, st>>>(g); });
   } else {
-    dim3 grid((g.M + 15) / 16, (g.N + 63) / 64);
+    dim3 grid((g.M + 15) / 16, (g.N + 63) / 64, nb);
     if (dtype == VRA_F32) launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<float, 1><<<grid, 256, 0, st>>>(g); });
     else launch_checked("stack gemm", [&] { stk_gemm_simple_kernel<uint16_t, 1><<<grid, 256, 0, st>>>(g); });
   }
@@ -997,7 +980,7 @@ void vra_stack_gemm(const StkGemmArgs& g, int dtype, int64_t stream) {
 
 void vra_stack_embed_sinpos(const uint32_t* ids, const int64_t* positions, const void* embed, const float* inv_freq, float* x, int T, int W, int V,
                             int dtype, int64_t stream) {
-  VRA_CHECK_ARG(ids && positions && embed && inv_freq && x && T > 0 && W > 0, "stack embed: null pointer or empty shape");
+  VRA_CHECK_ARG(ids && positions && embed && x && T > 0 && W > 0, "stack embed: null pointer or empty shape");
   if (dtype == VRA_F32)
     launch_checked("stack embed", [&] { stk_embed_sinpos_kernel<float><<<T, 256, 0, as_stream(stream)>>>(ids, positions, (const float*)embed, inv_freq, x, W, V); });
   else
@@ -1025,10 +1008,10 @@ void vra_stack_moe_sort(const int* pair_expert, const float* pair_weight, int P,
   });
 }
 
-void vra_stack_gated_act(const float* gu, void* out, int M, int F, float limit, float act_alpha, int dtype, int64_t stream) {
+void vra_stack_gated_act(const float* gu, void* out, int M, int F, float limit, float act_alpha, int dtype, int64_t stream, int act) {
   VRA_CHECK_ARG(gu && out && M > 0 && F > 0, "stack gated act: null pointer or empty shape");
-  if (dtype == VRA_F32) launch_checked("stack gated act", [&] { stk_gated_act_kernel<float><<<M, 256, 0, as_stream(stream)>>>(gu, (float*)out, F, limit, act_alpha); });
-  else launch_checked("stack gated act", [&] { stk_gated_act_kernel<uint16_t><<<M, 256, 0, as_stream(stream)>>>(gu, (uint16_t*)out, F, limit, act_alpha); });
+  if (dtype == VRA_F32) launch_checked("stack gated act", [&] { stk_gated_act_kernel<float><<<M, 256, 0, as_stream(stream)>>>(gu, (float*)out, F, limit, act_alpha, act); });
+  else launch_checked("stack gated act", [&] { stk_gated_act_kernel<uint16_t><<<M, 256, 0, as_stream(stream)>>>(gu, (uint16_t*)out, F, limit, act_alpha, act); });
 }
 
 void vra_stack_polynorm(const float* z, void* out, const float* coef, int M, int F, float eps, int dtype, int64_t stream) {
@@ -1072,7 +1055,8 @@ void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream) {
     else launch_checked("stack attention (decode)", [&] { stk_attn_decode_kernel<uint16_t><<<grid, 64 * STK_DW, lds, st>>>(a); });
     return;
   }
-  if (dtype == VRA_BF16 && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 256 && a.ldq % 8 == 0 && ((uintptr_t)a.q % 16 == 0) && a.BS % 32 == 0) {
+  if (dtype == VRA_BF16 && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 256 && a.ldq % 8 == 0 && ((uintptr_t)a.q % 16 == 0) && a.BS % 32 == 0 &&
+      a.k_ld % 8 == 0 && a.v_ld % 8 == 0 && ((uintptr_t)a.vc % 16 == 0)) {
     dim3 grid((a.max_q + 63) / 64, a.B, a.H);
 #define STK_PFM(DCV, VTV) launch_checked("stack attention (prefill, mfma)", [&] { stk_attn_prefill_mfma_kernel<DCV, VTV><<<grid, 256, 0, st>>>(a); })
     if (a.dim <= 64 && a.vdim <= 64) STK_PFM(2, 4);
@@ -1126,7 +1110,7 @@ extern "C" void vra_stack_op_moe_sort(const int32_t* pair_expert, const float* p
   vra_stack_moe_sort(pair_expert, pair_weight, P, top, n_groups, granule, max_rows, row_token, row_scale, row_pair, tile_group, stream);
 }
 extern "C" void vra_stack_op_gated_act(const float* gu, void* out, int32_t M, int32_t F, float limit, float act_alpha, int32_t dtype, int64_t stream) {
-  vra_stack_gated_act(gu, out, M, F, limit, act_alpha, dtype, stream);
+  vra_stack_gated_act(gu, out, M, F, limit, act_alpha, dtype, stream, 0);
 }
 extern "C" void vra_stack_op_polynorm(const float* z, void* out, const float* coef, int32_t M, int32_t F, float eps, int32_t dtype, int64_t stream) {
   vra_stack_polynorm(z, out, coef, M, F, eps, dtype, stream);

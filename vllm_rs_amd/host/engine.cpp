@@ -281,8 +281,9 @@ class Engine {
       h_swap_k_.assign(model_->kv_layers(), nullptr);
       h_swap_v_.assign(model_->kv_layers(), nullptr);
       for (int l = 0; l < model_->kv_layers(); l++)
-        if (hipHostMalloc(&h_swap_k_[l], (size_t)num_cpu_blocks_ * model_->k_block_bytes(l), hipHostMallocDefault) != hipSuccess ||
-            hipHostMalloc(&h_swap_v_[l], (size_t)num_cpu_blocks_ * model_->v_block_bytes(l), hipHostMallocDefault) != hipSuccess)
+        // (a layer whose values live in its key rows has no value blocks: 16 bytes stand in)
+        if (hipHostMalloc(&h_swap_k_[l], std::max<size_t>((size_t)num_cpu_blocks_ * model_->k_block_bytes(l), 16), hipHostMallocDefault) != hipSuccess ||
+            hipHostMalloc(&h_swap_v_[l], std::max<size_t>((size_t)num_cpu_blocks_ * model_->v_block_bytes(l), 16), hipHostMallocDefault) != hipSuccess)
           return fail("pinned alloc for the CPU swap space failed");
     }
     const size_t B = max_seqs_;

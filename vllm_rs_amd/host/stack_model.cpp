@@ -60,14 +60,29 @@ bool StackModel::parse_spec(const char* spec) {
       width_ = (int)num("width", 0), vocab_ = (int)num("vocab", 0), groups_ = (int)num("groups", 1);
       eps_ = (float)num("eps", 1e-6), residual_mult_ = (float)num("residual_mult", 1.0), logit_scale_ = (float)num("logit_scale", 1.0);
       pos_base_ = num("pos_base", 10000.0);
+      auto pick = [&](const char* k, const char* a, const char* b, int* out) {
+        const std::string v = f.count(k) ? f[k] : a;
+        if (v != a && v != b) return spec_error_ = std::string("layer stack spec: ") + k + " must be " + a + " or " + b, false;
+        *out = v == b;
+        return true;
+      };
+      if (!pick("block", "parallel", "sequential", &block_) || !pick("norm", "rms", "dyt", &norm_kind_) || !pick("pos", "sinusoid", "none", &pos_kind_)) return false;
     } else if (kind == "layer") {
       StackLayer L;
       L.heads = (int)num("heads", 0), L.kv_heads = (int)num("kv_heads", L.heads), L.dim = (int)num("dim", 0), L.vdim = (int)num("vdim", L.dim);
       L.scale = (float)num("scale", L.dim > 0 ? 1.0 / sqrt((double)L.dim) : 1.0), L.softcap = (float)num("softcap", 0.0);
       L.temp_coef = (float)num("temp_coef", 0.0), L.temp_every = (int)num("temp_every", 0), L.kv_from = (int)num("kv_from", -1);
+      const std::string mix = f.count("mixer") ? f["mixer"] : "attention";
+      L.mixer = mix == "latent" ? 1 : (mix == "sigmoid" ? 2 : 0);
+      if (mix != "attention" && mix != "latent" && mix != "sigmoid") return spec_error_ = "layer stack spec: unknown mixer " + mix, false;
+      L.weights_of = (int)num("weights_of", -1);
+      L.rot_dim = (int)num("rot_dim", 0), L.kv_rank = (int)num("kv_rank", 0), L.q_rank = (int)num("q_rank", 0), L.rot_dims = (int)num("rot_dims", L.rot_dim);
+      L.sink = (int)num("sink", 0), L.rot_base = num("rot_base", 10000.0), L.yarn_factor = num("yarn_factor", 0.0);
+      L.yarn_original = num("yarn_original", 0.0), L.yarn_fast = num("yarn_fast", 32.0), L.yarn_slow = num("yarn_slow", 1.0);
+      L.window = (int)num("window", 0), L.keep_first = (int)num("keep_first", 0), L.slope_exp = num("slope_exp", 0.0);
       const std::string mlp = f.count("mlp") ? f["mlp"] : "none";
-      L.mlp = mlp == "dense" ? 1 : (mlp == "moe" ? 2 : 0);
-      if (mlp != "dense" && mlp != "moe" && mlp != "none") return spec_error_ = "layer stack spec: unknown feed-forward kind " + mlp, false;
+      L.mlp = mlp == "dense" ? 1 : (mlp == "moe" ? 2 : (mlp == "gated" ? 3 : 0));
+      if (mlp != "dense" && mlp != "moe" && mlp != "none" && mlp != "gated") return spec_error_ = "layer stack spec: unknown feed-forward kind " + mlp, false;
       L.ff = (int)num("ff", 0), L.experts = (int)num("experts", 0), L.top = (int)num("top", 1), L.limit = (float)num("limit", 0.0);
       L.shared_ff = (int)num("shared_ff", 0), L.shared_limit = (float)num("shared_limit", 0.0);
       layers_.push_back(L);
@@ -82,8 +97,26 @@ bool StackModel::parse_spec(const char* spec) {
   for (size_t i = 0; i < layers_.size(); i++) {
     StackLayer& L = layers_[i];
     const std::string at = " (layer " + std::to_string(i) + ")";
-    if (L.heads <= 0 || L.kv_heads <= 0 || L.heads % L.kv_heads || L.dim <= 0 || L.vdim <= 0 || L.vdim > 256)
+    if (L.heads <= 0 || L.kv_heads <= 0 || L.heads % L.kv_heads || L.dim <= 0 || L.vdim <= 0 || (L.mixer == 0 && L.vdim > 256))
       return spec_error_ = "layer stack spec: heads must be a multiple of kv_heads, sizes positive, value size at most 256" + at, false;
+    if (L.mixer != 0 && block_ != 1) return spec_error_ = "layer stack spec: latent and sigmoid mixers run in sequential blocks" + at, false;
+    if (L.mixer == 0 && block_ != 0) return spec_error_ = "layer stack spec: the softmax mixer with temperature and cap runs in parallel blocks" + at, false;
+    if (L.mixer != 0 && L.kv_from >= 0) return spec_error_ = "layer stack spec: kv_from belongs to the softmax mixer" + at, false;
+    if (L.mixer == 1 && (L.kv_rank <= 0 || L.q_rank <= 0 || L.rot_dim < 0 || L.kv_rank > 256 || L.rot_dims < 0 || L.rot_dims > L.rot_dim || L.rot_dims % 2 ||
+                         (L.yarn_factor > 0.0 && (L.yarn_original <= 0.0 || L.yarn_fast <= 0.0 || L.yarn_slow <= 0.0))))
+      return spec_error_ = "layer stack spec: latent attention needs q_rank, 0 < kv_rank <= 256, an even rot_dims <= rot_dim" + at, false;
+    if ((L.mlp == 3) != (block_ == 1) && L.mlp != 0) return spec_error_ = "layer stack spec: the gated feed-forward belongs to sequential blocks, the others to parallel ones" + at, false;
+    if (L.weights_of >= 0) {
+      int root = L.weights_of;  // (a chain of references ends at a layer with tensors of its own)
+      for (size_t hop = 0; hop < layers_.size() && root >= 0 && root < (int)layers_.size() && layers_[root].weights_of >= 0; hop++) root = layers_[root].weights_of;
+      if (root < 0 || root >= (int)layers_.size() || root == (int)i || layers_[root].weights_of >= 0)
+        return spec_error_ = "layer stack spec: weights_of must name another layer with tensors of its own" + at, false;
+      L.weights_of = root;
+      const StackLayer& S = layers_[root];
+      if (S.mixer != L.mixer || S.heads != L.heads || S.kv_heads != L.kv_heads || S.dim != L.dim || S.vdim != L.vdim || S.rot_dim != L.rot_dim ||
+          S.kv_rank != L.kv_rank || S.q_rank != L.q_rank || S.mlp != L.mlp || S.ff != L.ff || S.kv_from >= 0 || L.kv_from >= 0)
+        return spec_error_ = "layer stack spec: a layer that shares weights has the shapes of the layer it names" + at, false;
+    }
     if (L.kv_from >= 0) {
       if (L.kv_from >= (int)i) return spec_error_ = "layer stack spec: kv_from must name an earlier layer" + at, false;
       const StackLayer& S = layers_[L.kv_from];
@@ -98,6 +131,10 @@ bool StackModel::parse_spec(const char* spec) {
     if (L.mlp == 1 && L.ff <= 0) return spec_error_ = "layer stack spec: dense feed-forward without ff" + at, false;
     if (L.mlp == 2 && (L.ff <= 0 || L.experts <= 0 || L.top < 1 || L.top > L.experts))
       return spec_error_ = "layer stack spec: mixture of experts needs ff, experts and 1 <= top <= experts" + at, false;
+    if (L.mlp == 3) {
+      if (L.ff <= 0) return spec_error_ = "layer stack spec: gated feed-forward without ff" + at, false;
+      L.shared_ff = L.ff;  // (laid out like a shared expert: gate / up rows interleaved, one weight set for all rows)
+    }
     L.ffp = round_up(L.ff, 16), L.sffp = round_up(L.shared_ff, 16);
   }
   return true;
@@ -165,6 +202,11 @@ float* StackModel::upload_f32(const HostTensor& t) {
   return (float*)upload(f.data(), n * 4);
 }
 
+float* StackModel::upload_floats(const std::vector<float>& v) {
+  weight_bytes_ += v.size() * 4;
+  return (float*)upload(v.data(), std::max<size_t>(v.size(), 1) * 4);
+}
+
 bool StackModel::finalize_weights() {
   if (finalized_) return true;
   if (!spec_error_.empty()) return error = spec_error_, false;
@@ -199,23 +241,124 @@ bool StackModel::finalize_weights() {
     memset(dst, 0, (size_t)W * fp * es);
     for (int r = 0; r < W; r++) memcpy(dst + (size_t)r * fp * es, d->data.data() + (size_t)r * f * es, (size_t)f * es);
   };
-  if (!up_mat("embed", vocab_, W, &embed_) || !up_mat("head", vocab_, W, &head_) || !up_vec("final.norm", W, &final_norm_)) return false;
+  auto up_scalar = [&](const std::string& name, float* dst) {
+    const HostTensor* t;
+    if (!need(name, 1, -1, &t)) return false;
+    float* d = upload_f32(*t);  // (kept on the device too: synthetic and loaded weights take one path)
+    if (!d) return false;
+    return hipMemcpy(dst, d, 4, hipMemcpyDeviceToHost) == hipSuccess;
+  };
+  auto up_norm = [&](const std::string& name, float** w, float** b, float* alpha) {
+    if (!up_vec(name, W, w)) return false;
+    if (norm_kind_ == 1 && (!up_vec(name + ".b", W, b) || !up_scalar(name + ".alpha", alpha))) return false;
+    return true;
+  };
+  // rows of several matrices of equal width under one another -> one device matrix
+  auto up_rows = [&](const std::vector<const HostTensor*>& parts, void** dst) {
+    std::vector<uint8_t> cat;
+    for (const HostTensor* t : parts) cat.insert(cat.end(), t->data.begin(), t->data.end());
+    weight_bytes_ += cat.size();
+    return (*dst = upload(cat.data(), cat.size())) != nullptr;
+  };
+  auto f32_of = [&](const HostTensor& t, std::vector<float>* out) {
+    const size_t n = t.data.size() / t.elem_bytes;
+    for (size_t i = 0; i < n; i++) {
+      float v;
+      if (t.elem_bytes == 4) memcpy(&v, t.data.data() + i * 4, 4);
+      else {
+        uint16_t b16;
+        memcpy(&b16, t.data.data() + i * 2, 2);
+        const uint32_t u = (uint32_t)b16 << 16;
+        memcpy(&v, &u, 4);
+      }
+      out->push_back(v);
+    }
+  };
+  if (!up_mat("embed", vocab_, W, &embed_) || !up_mat("head", vocab_, W, &head_) || !up_norm("final.norm", &final_norm_, &final_b_, &final_alpha_)) return false;
   for (size_t li = 0; li < layers_.size(); li++) {
     StackLayer& L = layers_[li];
+    if (L.weights_of >= 0) continue;
     const std::string p = "l" + std::to_string(li) + ".";
-    if (!up_vec(p + "norm1", W, &L.norm_w)) return false;
-    {  // q (| k | v) in one matrix: one launch projects them all
+    if (!up_norm(p + "norm1", &L.norm_w, &L.norm_b, &L.norm_alpha)) return false;
+    if (block_ == 1 && L.mlp != 0 && !up_norm(p + "norm2", &L.norm2_w, &L.norm2_b, &L.norm2_alpha)) return false;
+    if (L.mixer == 0) {  // q (| k | v) in one matrix: one launch projects them all
       const HostTensor *q, *k = nullptr, *v = nullptr;
       if (!need(p + "mix.q", L.nq(), W, &q) || !matrix(q)) return false;
       if (L.owns_cache && (!need(p + "mix.k", L.nk(), W, &k) || !need(p + "mix.v", L.nv(), W, &v) || !matrix(k) || !matrix(v))) return false;
-      std::vector<uint8_t> cat(q->data);
-      if (k) cat.insert(cat.end(), k->data.begin(), k->data.end()), cat.insert(cat.end(), v->data.begin(), v->data.end());
-      weight_bytes_ += cat.size();
-      if (!(L.qkv = upload(cat.data(), cat.size()))) return false;
+      std::vector<const HostTensor*> parts{q};
+      if (k) parts.push_back(k), parts.push_back(v);
+      if (!up_rows(parts, &L.qkv)) return false;
+    } else if (L.mixer == 1) {
+      // the two down-projections in one matrix [q latent | kv latent | rotated key part]; W_uk per head transposed, so that a query is
+      // carried into the latent's space (q_h . (W_uk_h c) = (W_uk_h^T q_h) . c) and the cache needs the latent alone
+      const HostTensor *dq, *dkv, *uk;
+      const int H = L.heads, qd = L.dim + L.rot_dim;
+      if (!need(p + "mix.dq", L.q_rank, W, &dq) || !need(p + "mix.dkv", L.kv_rank + L.rot_dim, W, &dkv) || !matrix(dq) || !matrix(dkv)) return false;
+      if (!up_rows({dq, dkv}, &L.qkv)) return false;
+      if (!up_vec(p + "mix.dq.norm", L.q_rank, &L.qn_w) || !up_vec(p + "mix.dkv.norm", L.kv_rank, &L.kn_w)) return false;
+      if (!up_mat(p + "mix.uq", (int64_t)H * qd, L.q_rank, &L.uq) || !up_mat(p + "mix.uv", (int64_t)H * L.vdim, L.kv_rank, &L.uv)) return false;
+      if (!need(p + "mix.uk", (int64_t)H * L.dim, L.kv_rank, &uk) || !matrix(uk)) return false;
+      std::vector<uint8_t> tr(uk->data.size());
+      for (int h = 0; h < H; h++)
+        for (int d = 0; d < L.dim; d++)
+          for (int r = 0; r < L.kv_rank; r++)
+            memcpy(tr.data() + (((size_t)h * L.kv_rank + r) * L.dim + d) * es, uk->data.data() + (((size_t)h * L.dim + d) * L.kv_rank + r) * es, es);
+      weight_bytes_ += tr.size();
+      if (!(L.ukt = upload(tr.data(), tr.size()))) return false;
+      if (L.sink && !up_vec(p + "mix.sink", H, &L.sink_w)) return false;
+      // rotary frequencies in f64, kept as hi + lo f32 pairs
+      L.rot_pairs = L.rot_dims / 2;
+      std::vector<float> fh(std::max(L.rot_pairs, 1)), fl(std::max(L.rot_pairs, 1));
+      const double dims = (double)L.rot_dims, lnb = log(L.rot_base);
+      double lo = 0.0, hi = 0.0;
+      L.rot_mag = 1.f;
+      if (L.yarn_factor > 0.0) {
+        auto turn_dim = [&](double turns) { return dims * log(L.yarn_original / (2.0 * M_PI * turns)) / (2.0 * lnb); };
+        lo = std::max(floor(turn_dim(L.yarn_fast)), 0.0), hi = std::min(ceil(turn_dim(L.yarn_slow)), dims - 1.0);
+        L.rot_mag = (float)(0.1 * log(L.yarn_factor) + 1.0);
+      }
+      for (int i = 0; i < L.rot_pairs; i++) {
+        double fr = pow(L.rot_base, -2.0 * (double)i / dims);
+        if (L.yarn_factor > 0.0) {
+          const double ramp = std::min(std::max(((double)i - lo) / std::max(hi - lo, 0.001), 0.0), 1.0);
+          fr = fr / L.yarn_factor * ramp + fr * (1.0 - ramp);
+        }
+        fh[i] = (float)fr, fl[i] = (float)(fr - (double)fh[i]);
+      }
+      if (!(L.freq_hi = upload_floats(fh)) || !(L.freq_lo = upload_floats(fl))) return false;
+    } else {
+      // q | k | v | output gate in one matrix, the biases of q, k, v as one f32 row (zeros under the gate)
+      const HostTensor *q, *k, *v, *g, *qb, *kb, *vb, *tk;
+      const int H = L.heads, ng = H * L.vdim;
+      if (!need(p + "mix.q", L.nq(), W, &q) || !need(p + "mix.k", L.nk(), W, &k) || !need(p + "mix.v", L.nv(), W, &v) || !need(p + "mix.g", ng, W, &g) ||
+          !matrix(q) || !matrix(k) || !matrix(v) || !matrix(g))
+        return false;
+      if (!up_rows({q, k, v, g}, &L.qkv)) return false;
+      if (!need(p + "mix.q.b", L.nq(), -1, &qb) || !need(p + "mix.k.b", L.nk(), -1, &kb) || !need(p + "mix.v.b", L.nv(), -1, &vb)) return false;
+      std::vector<float> bias;
+      f32_of(*qb, &bias), f32_of(*kb, &bias), f32_of(*vb, &bias);
+      bias.resize(bias.size() + ng, 0.f);
+      if (!(L.qkv_bias = upload_floats(bias))) return false;
+      if (!up_vec(p + "mix.q.norm", L.nq(), &L.qn_w) || !up_vec(p + "mix.k.norm", L.nk(), &L.kn_w) || !up_vec(p + "mix.pb", H, &L.head_bias)) return false;
+      if (!need(p + "mix.talk", H, H, &tk) || !(L.talk = upload_f32(*tk))) return false;
+      if (L.slope_exp != 0.0) {
+        std::vector<float> sl(H);
+        for (int h = 0; h < H; h++) sl[h] = (float)pow(2.0, -L.slope_exp * (double)(h + 1) / (double)H);
+        if (!(L.slopes = upload_floats(sl))) return false;
+      }
     }
     if (!up_mat(p + "mix.o", W, L.heads * L.vdim, &L.o)) return false;
     if (L.mlp == 1) {
       if (!up_mat(p + "mlp.up", L.ff, W, &L.up) || !up_mat(p + "mlp.down", W, L.ff, &L.down) || !up_vec(p + "mlp.act", 4, &L.act)) return false;
+    } else if (L.mlp == 3) {
+      const HostTensor *g, *u, *d;
+      if (!need(p + "mlp.gate", L.ff, W, &g) || !need(p + "mlp.up", L.ff, W, &u) || !need(p + "mlp.down", W, L.ff, &d) || !matrix(g) || !matrix(u) || !matrix(d))
+        return false;
+      std::vector<uint8_t> sgu((size_t)2 * L.sffp * W * es), sdn((size_t)W * L.sffp * es);
+      interleave(g, u, L.ff, L.sffp, sgu.data());
+      pad_cols(d, L.ff, L.sffp, sdn.data());
+      weight_bytes_ += sgu.size() + sdn.size();
+      if (!(L.s_gu = upload(sgu.data(), sgu.size())) || !(L.s_down = upload(sdn.data(), sdn.size()))) return false;
     } else if (L.mlp == 2) {
       const HostTensor *r, *sg = nullptr;
       if (!need(p + "mlp.router", L.experts, W, &r) || !matrix(r)) return false;
@@ -248,10 +391,18 @@ bool StackModel::finalize_weights() {
       }
     }
   }
+  // a layer that shares weights runs with the tensors of the layer it names and keeps a cache of its own
+  for (StackLayer& L : layers_) {
+    if (L.weights_of < 0) continue;
+    const int cache = L.cache, wo = L.weights_of;
+    const bool owns = L.owns_cache;
+    L = layers_[wo];
+    L.cache = cache, L.owns_cache = owns, L.weights_of = wo;
+  }
   // the angle of channel pair i is p * base^(-2i / width): the factor is formed in f64 and rounded once, the product is f32
   std::vector<float> inv((W + 1) / 2);
   for (size_t i = 0; i < inv.size(); i++) inv[i] = (float)pow(pos_base_, -2.0 * (double)i / (double)W);
-  if (!(inv_freq_ = (float*)upload(inv.data(), inv.size() * 4))) return false;
+  if (pos_kind_ == 0 && !(inv_freq_ = (float*)upload(inv.data(), inv.size() * 4))) return false;
   staged_.clear();
   finalized_ = hipDeviceSynchronize() == hipSuccess;
   if (!finalized_) error = "layer stack: device error while loading weights";
@@ -287,16 +438,39 @@ bool StackModel::init_synthetic(uint64_t seed) {
   const int W = width_;
   put("embed", vocab_, W, 0, 1.0);
   put("head", vocab_, W, 0, 1.0 / sqrt((double)W));
-  put("final.norm", W, 0, 1, 0.05);
+  auto put_norm = [&](const std::string& name) {
+    put(name, W, 0, 1, 0.05);
+    if (norm_kind_ == 1) put(name + ".b", W, 0, 0, 0.02), put(name + ".alpha", 1, 0, 0.5, 0.0);
+  };
+  put_norm("final.norm");
   for (size_t li = 0; li < layers_.size(); li++) {
     const StackLayer& L = layers_[li];
+    if (L.weights_of >= 0) continue;
     const std::string p = "l" + std::to_string(li) + ".";
     const double sw = 1.0 / sqrt((double)W);
-    put(p + "norm1", W, 0, 1, 0.05);
-    put(p + "mix.q", L.nq(), W, 0, sw);
-    if (L.owns_cache) put(p + "mix.k", L.nk(), W, 0, sw), put(p + "mix.v", L.nv(), W, 0, sw);
+    put_norm(p + "norm1");
+    if (block_ == 1 && L.mlp != 0) put_norm(p + "norm2");
+    if (L.mixer == 0) {
+      put(p + "mix.q", L.nq(), W, 0, sw);
+      if (L.owns_cache) put(p + "mix.k", L.nk(), W, 0, sw), put(p + "mix.v", L.nv(), W, 0, sw);
+    } else if (L.mixer == 1) {
+      put(p + "mix.dq", L.q_rank, W, 0, sw), put(p + "mix.dq.norm", L.q_rank, 0, 1, 0.05);
+      put(p + "mix.uq", (int64_t)L.heads * (L.dim + L.rot_dim), L.q_rank, 0, 1.0 / sqrt((double)L.q_rank));
+      put(p + "mix.dkv", L.kv_rank + L.rot_dim, W, 0, sw), put(p + "mix.dkv.norm", L.kv_rank, 0, 1, 0.05);
+      put(p + "mix.uk", (int64_t)L.heads * L.dim, L.kv_rank, 0, 1.0 / sqrt((double)L.kv_rank));
+      put(p + "mix.uv", (int64_t)L.heads * L.vdim, L.kv_rank, 0, 1.0 / sqrt((double)L.kv_rank));
+      if (L.sink) put(p + "mix.sink", L.heads, 0, 0, 1.0);
+    } else {
+      put(p + "mix.q", L.nq(), W, 0, sw), put(p + "mix.k", L.nk(), W, 0, sw), put(p + "mix.v", L.nv(), W, 0, sw);
+      put(p + "mix.g", (int64_t)L.heads * L.vdim, W, 0, sw);
+      put(p + "mix.q.b", L.nq(), 0, 0, 0.02), put(p + "mix.k.b", L.nk(), 0, 0, 0.02), put(p + "mix.v.b", L.nv(), 0, 0, 0.02);
+      put(p + "mix.q.norm", L.nq(), 0, 1, 0.05), put(p + "mix.k.norm", L.nk(), 0, 1, 0.05);
+      put(p + "mix.pb", L.heads, 0, -3.0, 0.5), put(p + "mix.talk", L.heads, L.heads, 1.0 / L.heads, 0.1 / L.heads);
+    }
     put(p + "mix.o", W, L.heads * L.vdim, 0, 1.0 / sqrt((double)L.heads * L.vdim));
-    if (L.mlp == 1) {
+    if (L.mlp == 3) {
+      put(p + "mlp.gate", L.ff, W, 0, sw), put(p + "mlp.up", L.ff, W, 0, sw), put(p + "mlp.down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
+    } else if (L.mlp == 1) {
       put(p + "mlp.up", L.ff, W, 0, sw), put(p + "mlp.down", W, L.ff, 0, 1.0 / sqrt((double)L.ff));
       HostTensor a;
       a.elem_bytes = 4, a.shape = {4};
@@ -323,11 +497,11 @@ bool StackModel::init_synthetic(uint64_t seed) {
 // ---------------------------------------------------------------------------------------------
 size_t StackModel::k_block_bytes(int c) const {
   const StackLayer& L = layers_[cache_layer_[c]];
-  return (size_t)ec_.block_size * L.nk() * es_;
+  return (size_t)ec_.block_size * L.k_row() * es_;
 }
 size_t StackModel::v_block_bytes(int c) const {
   const StackLayer& L = layers_[cache_layer_[c]];
-  return (size_t)ec_.block_size * L.nv() * es_;
+  return (size_t)ec_.block_size * L.v_row() * es_;
 }
 int64_t StackModel::kv_bytes_per_block() const {
   int64_t b = 0;
@@ -352,9 +526,15 @@ bool StackModel::init_buffers(int max_tokens, int max_seqs) {
   max_tokens_ = max_tokens, max_seqs_ = max_seqs;
   const size_t T = max_tokens, W = width_;
   size_t nqkv = 0, nattn = 0, zc = 0, actc = 0, top = 0, experts = 0;
+  size_t nqa = 0;
   for (const StackLayer& L : layers_) {
-    nqkv = std::max(nqkv, (size_t)L.nqkv()), nattn = std::max(nattn, (size_t)L.heads * L.vdim);
+    // softmax / sigmoid: the joint projection in the model's type; latent: q, later the heads' values (the joint projection is f32 in z_)
+    nqkv = std::max(nqkv, L.mixer == 0 ? (size_t)L.nqkv() : std::max((size_t)L.nq(), (size_t)L.heads * L.vdim));
+    nattn = std::max(nattn, (size_t)L.heads * (L.mixer == 1 ? L.kv_rank : L.vdim));
+    if (L.mixer == 1) nqa = std::max(nqa, (size_t)L.heads * (L.kv_rank + L.rot_dim)), actc = std::max(actc, T * L.q_rank);
+    if (L.mixer != 0) zc = std::max(zc, T * L.nqkv());
     if (L.mlp == 2) top = std::max(top, (size_t)L.top), experts = std::max(experts, (size_t)L.experts);
+    if (L.mlp == 3) zc = std::max(zc, T * 2 * L.sffp), actc = std::max(actc, T * L.sffp);
   }
   max_rows_ = (int)round_up((int)(T * std::max<size_t>(top, 1) + experts * 63), 64);
   for (const StackLayer& L : layers_) {
@@ -370,7 +550,7 @@ bool StackModel::init_buffers(int max_tokens, int max_seqs) {
   if (!(x_ = (float*)dalloc(T * W * 4)) || !(o_ = (float*)dalloc(T * W * 4)) || !(h_ = dalloc(T * W * es_)) || !(qkv_ = dalloc(T * nqkv * es_)) ||
       !(attn_ = dalloc(T * nattn * es_)) || !(z_ = (float*)dalloc(std::max<size_t>(zc, 4) * 4)) || !(act_ = dalloc(std::max<size_t>(actc, 4) * es_)) ||
       !(pair_out_ = (float*)dalloc(T * std::max<size_t>(top, 1) * W * 4)) || !(sh_ = (float*)dalloc(T * W * 4)) || !(xl_ = (float*)dalloc(R * W * 4)) ||
-      !(hl_ = dalloc(R * W * es_)) || !(logits_ = (float*)dalloc(R * (size_t)vocab_ * 4)))
+      !(hl_ = dalloc(R * W * es_)) || !(logits_ = (float*)dalloc(R * (size_t)vocab_ * 4)) || !(qa_ = dalloc(std::max<size_t>(T * nqa, 4) * es_)))
     return false;
   const size_t P = T * std::max<size_t>(top, 1);
   if (!(pair_expert_ = (int*)dalloc(P * 4)) || !(pair_weight_ = (float*)dalloc(P * 4)) || !(gate_ = (float*)dalloc(T * 4)) ||
@@ -397,12 +577,12 @@ static bool take_stack_err(std::string& error, const char* where) {
 // bf16: the activation is the epilogue of the gate / up launch; f32: product, activation and product as three launches
 bool StackModel::expert_pair(const void* a, int lda, const void* w_gu, int64_t gu_stride, const void* w_down, int64_t down_stride, int rows, int fp,
                              int f, float limit, const int* tile_group, int granule, const int* a_row, const float* a_scale, const int* out_row,
-                             float* out, int64_t stream) {
+                             float* out, int64_t stream, int act) {
   const int W = width_;
   StkGemmArgs g;
   g.a = a, g.lda = lda, g.w = w_gu, g.w_group_stride = gu_stride, g.M = rows, g.N = 2 * fp, g.K = W;
   g.tile_group = tile_group, g.granule = granule, g.a_row = a_row, g.a_scale = a_scale;
-  g.limit = limit;
+  g.limit = limit, g.act = act;
   const bool fused = dt_ == VRA_BF16 && W % 8 == 0 && lda % 8 == 0;
   if (fused) {
     g.epi = 1, g.out = act_, g.ldo = fp;
@@ -410,7 +590,7 @@ bool StackModel::expert_pair(const void* a, int lda, const void* w_gu, int64_t g
   } else {
     g.out = z_, g.ldo = 2 * fp, g.out_f32 = 1;
     vra_stack_gemm(g, dt_, stream);
-    vra_stack_gated_act(z_, act_, rows, f, limit, 1.702f, dt_, stream);
+    vra_stack_gated_act(z_, act_, rows, f, limit, 1.702f, dt_, stream, act);
   }
   StkGemmArgs d;
   d.a = act_, d.lda = fp, d.w = w_down, d.w_group_stride = down_stride, d.M = rows, d.N = W, d.K = fp;
@@ -454,6 +634,104 @@ bool StackModel::feed_forward(const StackLayer& L, int T, int64_t stream) {
   return !take_stack_err(error, "residual");
 }
 
+// h = norm(x + add) with x updated in place (add null: x as it is); sequential blocks norm every sub-block's input
+bool StackModel::norm_into_h(const float* w, const float* b, float alpha, const float* add, float* x, void* h, int T, int64_t stream) {
+  if (norm_kind_ == 1) {
+    vra_stack_dyt(x, add, w, b, alpha, h, T, width_, dt_, stream);
+  } else {
+    if (add) vra_stack_residual_combine(x, add, nullptr, 0, nullptr, nullptr, 1.f, T, width_, stream);
+    StkNormArgs n;
+    n.x = x, n.w = w, n.h = h, n.T = T, n.W = width_, n.groups = groups_, n.eps = eps_;
+    vra_stack_group_norm(n, dt_, stream);
+  }
+  return !take_stack_err(error, "norm");
+}
+
+// causal softmax attention with its own (or a borrowed) key / value cache: h_ -> o_ (f32 [T, width])
+bool StackModel::mixer_softmax(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, B = md.n_seqs, W = width_;
+  // q (| k | v) in one launch
+  const int nqkv = L.nqkv();
+  StkGemmArgs p;
+  p.a = h_, p.lda = W, p.w = L.qkv, p.M = T, p.N = nqkv, p.K = W, p.out = qkv_, p.ldo = nqkv;
+  vra_stack_gemm(p, dt_, stream);
+  if (L.owns_cache)
+    vra_stack_kv_store((const char*)qkv_ + (size_t)L.nq() * es_, (const char*)qkv_ + (size_t)(L.nq() + L.nk()) * es_, nqkv, kc_[L.cache], vc_[L.cache],
+                       md.slot_mapping, T, L.nk(), L.nv(), dt_, stream);
+  StkAttnArgs a;
+  a.q = qkv_, a.ldq = nqkv, a.out = attn_, a.kc = kc_[L.cache], a.vc = vc_[L.cache];
+  a.positions = md.positions, a.block_tables = md.block_tables, a.context_lens = md.context_lens;
+  a.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
+  a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = L.heads, a.G = L.kv_heads, a.dim = L.dim, a.vdim = L.vdim;
+  a.BS = ec_.block_size, a.max_blocks = md.max_blocks;
+  a.scale = L.scale, a.softcap = L.softcap, a.temp_coef = L.temp_coef, a.temp_every = L.temp_every;
+  vra_stack_attention(a, dt_, stream);
+  StkGemmArgs o;
+  o.a = attn_, o.lda = L.heads * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = L.heads * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;
+  vra_stack_gemm(o, dt_, stream);
+  return !take_stack_err(error, "mixer");
+}
+
+// Latent attention in its absorbed form: the cache row of a token is [normed kv latent | rotated key part]; a head's query becomes
+// [W_uk_h^T q_h | rot(q_h's rotated part)], so the scores are plain dot products with the cache rows of ONE shared key/value head, the
+// values are the latents themselves, and W_uv_h is applied to the weighted sum.
+bool StackModel::mixer_latent(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, B = md.n_seqs, W = width_, H = L.heads, qd = L.dim + L.rot_dim, kd = L.kv_rank + L.rot_dim;
+  StkGemmArgs d;  // both down-projections, f32 out: the norms read unrounded values
+  d.a = h_, d.lda = W, d.w = L.qkv, d.M = T, d.N = L.nqkv(), d.K = W, d.out = z_, d.ldo = L.nqkv(), d.out_f32 = 1;
+  vra_stack_gemm(d, dt_, stream);
+  StkLatentPrepArgs lp;
+  lp.raw = z_, lp.ld = L.nqkv(), lp.q_rank = L.q_rank, lp.kv_rank = L.kv_rank, lp.rot_dim = L.rot_dim, lp.qn_w = L.qn_w, lp.kvn_w = L.kn_w, lp.eps = eps_;
+  lp.cq = act_, lp.cache = kc_[L.cache], lp.cache_ld = kd, lp.slots = md.slot_mapping, lp.positions = md.positions, lp.T = T;
+  lp.rot.freq_hi = L.freq_hi, lp.rot.freq_lo = L.freq_lo, lp.rot.pairs = L.rot_pairs, lp.rot.mag = L.rot_mag;
+  vra_stack_latent_prep(lp, dt_, stream);
+  StkGemmArgs uq;
+  uq.a = act_, uq.lda = L.q_rank, uq.w = L.uq, uq.M = T, uq.N = H * qd, uq.K = L.q_rank, uq.out = qkv_, uq.ldo = H * qd;
+  vra_stack_gemm(uq, dt_, stream);
+  if (L.rot_dim > 0) vra_stack_rope_heads(qkv_, H * qd, qd, L.dim, qa_, H * kd, kd, L.kv_rank, L.rot_dim, H, md.positions, lp.rot, T, dt_, stream);
+  StkGemmArgs ab;  // per head: [T, dim] x W_uk_h -> [T, kv_rank]
+  ab.a = qkv_, ab.lda = H * qd, ab.a_batch_stride = qd, ab.w = L.ukt, ab.w_batch_stride = (int64_t)L.kv_rank * L.dim, ab.batch = H;
+  ab.M = T, ab.N = L.kv_rank, ab.K = L.dim, ab.out = qa_, ab.ldo = H * kd, ab.out_batch_stride = kd;
+  vra_stack_gemm(ab, dt_, stream);
+  StkAttnArgs a;
+  a.q = qa_, a.ldq = H * kd, a.out = attn_, a.kc = kc_[L.cache], a.vc = kc_[L.cache], a.k_ld = kd, a.v_ld = kd, a.sink = L.sink ? L.sink_w : nullptr;
+  a.positions = md.positions, a.block_tables = md.block_tables, a.context_lens = md.context_lens;
+  a.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
+  a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = H, a.G = 1, a.dim = kd, a.vdim = L.kv_rank;
+  a.BS = ec_.block_size, a.max_blocks = md.max_blocks, a.scale = L.scale;
+  vra_stack_attention(a, dt_, stream);
+  StkGemmArgs uv;  // per head: [T, kv_rank] x W_uv_h^T -> [T, vdim]
+  uv.a = attn_, uv.lda = H * L.kv_rank, uv.a_batch_stride = L.kv_rank, uv.w = L.uv, uv.w_batch_stride = (int64_t)L.vdim * L.kv_rank, uv.batch = H;
+  uv.M = T, uv.N = L.vdim, uv.K = L.kv_rank, uv.out = qkv_, uv.ldo = H * L.vdim, uv.out_batch_stride = L.vdim;
+  vra_stack_gemm(uv, dt_, stream);
+  StkGemmArgs o;
+  o.a = qkv_, o.lda = H * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = H * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;
+  vra_stack_gemm(o, dt_, stream);
+  return !take_stack_err(error, "latent attention");
+}
+
+// sigmoid attention: q | k | v | gate in one launch (biases in its epilogue, f32 out), the two whole-projection norms and the cache rows
+// in one launch, then the attention with the gate in its epilogue
+bool StackModel::mixer_sigmoid(const StackLayer& L, const InputMetadata& md, int64_t stream) {
+  const int T = md.n_tokens, B = md.n_seqs, W = width_, n4 = L.nqkv();
+  StkGemmArgs p;
+  p.a = h_, p.lda = W, p.w = L.qkv, p.bias = L.qkv_bias, p.M = T, p.N = n4, p.K = W, p.out = z_, p.ldo = n4, p.out_f32 = 1;
+  vra_stack_gemm(p, dt_, stream);
+  vra_stack_qk_norm_store(z_, n4, L.nq(), L.nk(), L.nv(), L.qn_w, L.kn_w, eps_, qkv_, kc_[L.cache], vc_[L.cache], md.slot_mapping, T, dt_, stream);
+  StkSigAttnArgs a;
+  a.q = qkv_, a.ldq = L.nq(), a.out = attn_, a.kc = kc_[L.cache], a.vc = vc_[L.cache];
+  a.positions = md.positions, a.block_tables = md.block_tables, a.context_lens = md.context_lens;
+  a.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
+  a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = L.heads, a.G = L.kv_heads, a.dim = L.dim, a.vdim = L.vdim;
+  a.BS = ec_.block_size, a.max_blocks = md.max_blocks, a.scale = L.scale, a.window = L.window, a.keep_first = L.keep_first;
+  a.slopes = L.slopes, a.head_bias = L.head_bias, a.talk = L.talk, a.gate = z_ + L.nq() + L.nk() + L.nv(), a.gate_ld = n4;
+  vra_stack_sigmoid_attention(a, dt_, stream);
+  StkGemmArgs o;
+  o.a = attn_, o.lda = L.heads * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = L.heads * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;
+  vra_stack_gemm(o, dt_, stream);
+  return !take_stack_err(error, "sigmoid attention");
+}
+
 bool StackModel::forward(const InputMetadata& md, int64_t stream, uint32_t* tokens) {
   if (!finalized_) return error = "forward before the weights are complete", false;
   const int T = md.n_tokens, B = md.n_seqs, W = width_;
@@ -469,39 +747,38 @@ bool StackModel::forward(const InputMetadata& md, int64_t stream, uint32_t* toke
     }
     trace_bytes_ = need_b;
   }
-  vra_stack_embed_sinpos(md.input_ids, md.positions, embed_, inv_freq_, x_, T, W, vocab_, dt_, stream);
+  vra_stack_embed_sinpos(md.input_ids, md.positions, embed_, pos_kind_ == 0 ? inv_freq_ : nullptr, x_, T, W, vocab_, dt_, stream);
   if (take_stack_err(error, "embedding")) return false;
+  // sequential blocks: the output of a sub-block is added to the residual inside the launch of the next norm (`pending`)
+  const float* pending = nullptr;
   for (size_t li = 0; li < layers_.size(); li++) {
     const StackLayer& L = layers_[li];
-    // h = norm(x); a mixture-of-experts layer's router (and its shared expert's gate) reads h inside the same launch
-    StkNormArgs n;
-    n.x = x_, n.w = L.norm_w, n.h = h_, n.T = T, n.W = W, n.groups = groups_, n.eps = eps_;
-    if (L.mlp == 2) {
-      n.router_w = L.router, n.n_router = L.experts, n.top = L.top, n.gate_row = L.shared_ff > 0;
-      n.pair_expert = pair_expert_, n.pair_weight = pair_weight_, n.gate_out = gate_;
+    if (block_ == 0) {
+      // h = norm(x); a mixture-of-experts layer's router (and its shared expert's gate) reads h inside the same launch
+      StkNormArgs n;
+      n.x = x_, n.w = L.norm_w, n.h = h_, n.T = T, n.W = W, n.groups = groups_, n.eps = eps_;
+      if (L.mlp == 2) {
+        n.router_w = L.router, n.n_router = L.experts, n.top = L.top, n.gate_row = L.shared_ff > 0;
+        n.pair_expert = pair_expert_, n.pair_weight = pair_weight_, n.gate_out = gate_;
+      }
+      vra_stack_group_norm(n, dt_, stream);
+      if (!mixer_softmax(L, md, stream)) return false;
+      if (!feed_forward(L, T, stream)) return false;
+    } else {
+      if (!norm_into_h(L.norm_w, L.norm_b, L.norm_alpha, pending, x_, h_, T, stream)) return false;
+      if (!(L.mixer == 1 ? mixer_latent(L, md, stream) : (L.mixer == 2 ? mixer_sigmoid(L, md, stream) : mixer_softmax(L, md, stream)))) return false;
+      pending = o_;
+      if (L.mlp == 3) {
+        if (!norm_into_h(L.norm2_w, L.norm2_b, L.norm2_alpha, pending, x_, h_, T, stream)) return false;
+        if (!expert_pair(h_, W, L.s_gu, 0, L.s_down, 0, T, L.sffp, L.ff, 0.f, nullptr, 0, nullptr, nullptr, nullptr, pair_out_, stream, 1)) return false;
+        pending = pair_out_;
+      }
+      if (trace_on_ || li + 1 == layers_.size()) {
+        vra_stack_residual_combine(x_, pending, nullptr, 0, nullptr, nullptr, 1.f, T, W, stream);
+        pending = nullptr;
+        if (take_stack_err(error, "residual")) return false;
+      }
     }
-    vra_stack_group_norm(n, dt_, stream);
-    // q (| k | v) in one launch
-    const int nqkv = L.nqkv();
-    StkGemmArgs p;
-    p.a = h_, p.lda = W, p.w = L.qkv, p.M = T, p.N = nqkv, p.K = W, p.out = qkv_, p.ldo = nqkv;
-    vra_stack_gemm(p, dt_, stream);
-    if (L.owns_cache)
-      vra_stack_kv_store((const char*)qkv_ + (size_t)L.nq() * es_, (const char*)qkv_ + (size_t)(L.nq() + L.nk()) * es_, nqkv, kc_[L.cache], vc_[L.cache],
-                         md.slot_mapping, T, L.nk(), L.nv(), dt_, stream);
-    StkAttnArgs a;
-    a.q = qkv_, a.ldq = nqkv, a.out = attn_, a.kc = kc_[L.cache], a.vc = vc_[L.cache];
-    a.positions = md.positions, a.block_tables = md.block_tables, a.context_lens = md.context_lens;
-    a.cu_q = md.is_prefill ? md.cu_seqlens_q : nullptr;
-    a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = L.heads, a.G = L.kv_heads, a.dim = L.dim, a.vdim = L.vdim;
-    a.BS = ec_.block_size, a.max_blocks = md.max_blocks;
-    a.scale = L.scale, a.softcap = L.softcap, a.temp_coef = L.temp_coef, a.temp_every = L.temp_every;
-    vra_stack_attention(a, dt_, stream);
-    StkGemmArgs o;
-    o.a = attn_, o.lda = L.heads * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = L.heads * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;
-    vra_stack_gemm(o, dt_, stream);
-    if (take_stack_err(error, "mixer")) return false;
-    if (!feed_forward(L, T, stream)) return false;
     if (trace_on_ && hipMemcpyAsync(trace_ + li * (size_t)T * W, x_, (size_t)T * W * 4, hipMemcpyDeviceToDevice, st) != hipSuccess)
       return error = "layer trace copy failed", false;
   }
@@ -517,9 +794,14 @@ bool StackModel::forward(const InputMetadata& md, int64_t stream, uint32_t* toke
   } else if (rows > logit_rows_cap_) {
     return error = "forward: more logit rows than the logits buffer holds", false;
   }
-  StkNormArgs fn;
-  fn.x = xin, fn.w = final_norm_, fn.h = hl_, fn.T = rows, fn.W = W, fn.groups = groups_, fn.eps = eps_;
-  vra_stack_group_norm(fn, dt_, stream);
+  if (norm_kind_ == 1) {
+    // (the gathered rows are a copy: the kernel may read them through a non-const pointer, it adds nothing)
+    vra_stack_dyt(const_cast<float*>(xin), nullptr, final_norm_, final_b_, final_alpha_, hl_, rows, W, dt_, stream);
+  } else {
+    StkNormArgs fn;
+    fn.x = xin, fn.w = final_norm_, fn.h = hl_, fn.T = rows, fn.W = W, fn.groups = groups_, fn.eps = eps_;
+    vra_stack_group_norm(fn, dt_, stream);
+  }
   StkGemmArgs hd;
   hd.a = hl_, hd.lda = W, hd.w = head_, hd.M = rows, hd.N = vocab_, hd.K = W, hd.out = logits_, hd.ldo = vocab_, hd.out_f32 = 1, hd.alpha = logit_scale_;
   vra_stack_gemm(hd, dt_, stream);

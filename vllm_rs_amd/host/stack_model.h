@@ -1,16 +1,29 @@
-// stack_model.h — a decoder described by a LIST OF LAYERS instead of one fixed block: every layer names its mixer (attention with its own
-// head counts, score scale, soft cap, query temperature, optionally reading another layer's keys and values) and its feed-forward
-// (none, dense with a PolyNorm activation, or a mixture of clamped gated experts with a sigmoid router and a gated shared expert);
-// layers are parallel blocks  x <- x + m * (mixer(h) + ff(h)),  h = grouped RMS norm of x;  positions enter as a sinusoidal vector added
-// to the embedding.  The Ditilix design is such a list (vllm_rs_amd/checkpoint.py turns its config.json into the spec text below).
+// stack_model.h — a decoder described by a LIST OF LAYERS instead of one fixed block.  Every layer names its mixer and its feed-forward
+// with all sizes and constants; the record of the whole stack names the block form, the norm and how positions enter.
 //
-// Precision: the residual stream, norms, router, attention scores and weights are f32; projections, the cache and activations are
-// bf16 (f32 accumulation) or, for a VRA_F32 model, f32 throughout.
+//   block   parallel:    x <- x + m * (mixer(h) + ff(h)),  h = norm(x)                      (Ditilix)
+//           sequential:  x <- x + mixer(norm1(x)),  x <- x + ff(norm2(x))                   (Gaperax)
+//   norm    rms: RMS norm over `groups` equal parts of the width;  dyt: Dynamic Tanh  tanh(alpha x) w + b  (no statistics)
+//   pos     sinusoid: a position vector added to the embedding;  none: positions enter inside the mixers
+//   mixer   attention: causal softmax, query temperature, soft cap, grouped key/value heads, optionally another layer's keys / values
+//           latent:    queries and keys / values through low-rank latents, a rotated key part shared by the heads (rotary with optional
+//                      YaRN scaling), a softmax sink per head; the cache holds one row [latent | rotated part] per token and the
+//                      up-projections are absorbed: q' = [W_uk_h^T q_h | rot(q_h)], values = the latent, W_uv_h after the sum over keys
+//           sigmoid:   biased q / k / v, one RMS norm over all of q and all of k, weights sigmoid(score - slope_h * distance + bias_h)
+//                      without normalisation, a window that keeps the first tokens, heads mixed by a matrix, a sigmoid output gate
+//   mlp     none | dense (PolyNorm activation) | moe (sigmoid router, clamped gated experts, gated shared expert) | gated (gelu_tanh(gate) * up)
+//   weights_of=j: the layer runs with layer j's tensors and a cache of its own
+// vllm_rs_amd/checkpoint.py turns a design's config.json into the spec text below.
+//
+// Precision: the residual stream, norms, router, rotary angles, attention scores and weights are f32; projections, the cache and
+// activations are bf16 (f32 accumulation) or, for a VRA_F32 model, f32 throughout.
 //
 // Spec text, one record per line, `key=value` fields:
-//   stack width=.. vocab=.. eps=.. groups=.. residual_mult=.. logit_scale=.. pos_base=..
-//   layer heads=.. kv_heads=.. dim=.. vdim=.. scale=.. softcap=.. temp_coef=.. temp_every=.. kv_from=.. mlp=none|dense|moe ff=..
-//         experts=.. top=.. limit=.. shared_ff=.. shared_limit=..
+//   stack width=.. vocab=.. eps=.. groups=.. residual_mult=.. logit_scale=.. pos_base=.. block=.. norm=.. pos=..
+//   layer mixer=.. heads=.. kv_heads=.. dim=.. vdim=.. scale=.. softcap=.. temp_coef=.. temp_every=.. kv_from=.. weights_of=..
+//         rot_dim=.. kv_rank=.. q_rank=.. rot_dims=.. rot_base=.. yarn_factor=.. yarn_original=.. yarn_fast=.. yarn_slow=.. sink=0|1
+//         window=.. keep_first=.. slope_exp=..
+//         mlp=none|dense|moe|gated ff=.. experts=.. top=.. limit=.. shared_ff=.. shared_limit=..
 #pragma once
 #include <map>
 #include <string>
@@ -21,31 +34,57 @@
 namespace vra {
 
 struct StackLayer {
-  // mixer
-  int heads = 0, kv_heads = 0, dim = 0, vdim = 0, temp_every = 0, kv_from = -1;
+  // mixer: 0 softmax attention, 1 latent attention, 2 sigmoid attention
+  int mixer = 0;
+  int heads = 0, kv_heads = 0, dim = 0, vdim = 0, temp_every = 0, kv_from = -1, weights_of = -1;
   float scale = 1.f, softcap = 0.f, temp_coef = 0.f;
-  // feed-forward: 0 none, 1 dense (PolyNorm), 2 mixture of experts
+  // latent attention
+  int rot_dim = 0, kv_rank = 0, q_rank = 0, rot_dims = 0, sink = 0;
+  double rot_base = 10000.0, yarn_factor = 0.0, yarn_original = 0.0, yarn_fast = 32.0, yarn_slow = 1.0;
+  // sigmoid attention: window <= 0 = every earlier token; slope_h = 2^(-slope_exp (h + 1) / heads), 0 = no distance penalty
+  int window = 0, keep_first = 0;
+  double slope_exp = 0.0;
+  // feed-forward: 0 none, 1 dense (PolyNorm), 2 mixture of experts, 3 gated dense (gelu_tanh(gate) * up)
   int mlp = 0, ff = 0, experts = 0, top = 0, shared_ff = 0;
   float limit = 0.f, shared_limit = 0.f;
   // derived
   int cache = -1;          // index of the paged cache this layer reads (its own, or the one of layer kv_from)
   bool owns_cache = false;
-  int ffp = 0, sffp = 0;   // expert / shared widths rounded up to 16 (zero rows and columns)
-  int nq() const { return heads * dim; }
+  int ffp = 0, sffp = 0;   // expert / shared (or gated dense) widths rounded up to 16 (zero rows and columns)
+  int nq() const { return heads * (mixer == 1 ? dim + rot_dim : dim); }
   int nk() const { return kv_heads * dim; }
   int nv() const { return kv_heads * vdim; }
-  int nqkv() const { return nq() + (owns_cache ? nk() + nv() : 0); }
+  // columns of the joint input projection: q (| k | v) of softmax attention, q | k | v | gate of sigmoid attention, the three latents
+  int nqkv() const {
+    if (mixer == 1) return q_rank + kv_rank + rot_dim;
+    if (mixer == 2) return nq() + nk() + nv() + heads * vdim;
+    return nq() + (owns_cache ? nk() + nv() : 0);
+  }
+  // elements of one token's cache rows
+  int k_row() const { return mixer == 1 ? kv_rank + rot_dim : nk(); }
+  int v_row() const { return mixer == 1 ? 0 : nv(); }
   // device weights
   float* norm_w = nullptr;
-  void* qkv = nullptr;     // [nq (+ nk + nv), width]
+  float *norm_b = nullptr, *norm2_w = nullptr, *norm2_b = nullptr;  // Dynamic Tanh: offsets, and the second norm of a sequential block
+  float norm_alpha = 1.f, norm2_alpha = 1.f;
+  void* qkv = nullptr;     // [nqkv(), width]
+  float* qkv_bias = nullptr;  // sigmoid attention: f32 [nqkv()] (zeros for the gate rows)
   void* o = nullptr;       // [width, heads * vdim]
+  void* uq = nullptr;      // latent: [heads * (dim + rot_dim), q_rank]
+  void* ukt = nullptr;     // latent: [heads][kv_rank][dim] — W_uk of a head, transposed
+  void* uv = nullptr;      // latent: [heads * vdim, kv_rank]
+  float *qn_w = nullptr, *kn_w = nullptr;  // latent: norms of the two latents; sigmoid: norms over all of q / all of k
+  float *sink_w = nullptr, *freq_hi = nullptr, *freq_lo = nullptr;
+  int rot_pairs = 0;
+  float rot_mag = 1.f;
+  float *talk = nullptr, *head_bias = nullptr, *slopes = nullptr;
   void* up = nullptr;      // dense [ff, width]
   void* down = nullptr;    // dense [width, ff]
   float* act = nullptr;    // PolyNorm a, b, c, e
   void* router = nullptr;  // [experts (+ 1: the shared expert's gate), width]
   void* e_gu = nullptr;    // [experts][2 * ffp][width], gate / up rows interleaved in blocks of 16
   void* e_down = nullptr;  // [experts][width][ffp]
-  void* s_gu = nullptr;    // [2 * sffp][width]
+  void* s_gu = nullptr;    // [2 * sffp][width]  (shared expert, or the gated dense feed-forward)
   void* s_down = nullptr;  // [width][sffp]
 };
 
@@ -88,15 +127,21 @@ class StackModel : public ModelBase {
   float* upload_f32(const HostTensor& t);
   bool parse_spec(const char* spec);
   bool feed_forward(const StackLayer& L, int T, int64_t stream);
+  bool mixer_softmax(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool mixer_latent(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  bool mixer_sigmoid(const StackLayer& L, const InputMetadata& md, int64_t stream);
+  float* upload_floats(const std::vector<float>& v);
+  bool norm_into_h(const float* w, const float* b, float alpha, const float* add, float* x, void* h, int T, int64_t stream);
   bool expert_pair(const void* a, int lda, const void* w_gu, int64_t gu_stride, const void* w_down, int64_t down_stride, int rows, int fp, int f,
                    float limit, const int* tile_group, int granule, const int* a_row, const float* a_scale, const int* out_row, float* out,
-                   int64_t stream);
+                   int64_t stream, int act = 0);
   vra_model_config mc_;
   vra_engine_config ec_;
   std::string spec_error_;
   int dt_ = 0;
   size_t es_ = 2;
   int width_ = 0, vocab_ = 0, groups_ = 1;
+  int block_ = 0, norm_kind_ = 0, pos_kind_ = 0;  // 0 parallel / rms / sinusoid, 1 sequential / dyt / none
   float eps_ = 1e-6f, residual_mult_ = 1.f, logit_scale_ = 1.f;
   double pos_base_ = 10000.0;
   std::vector<StackLayer> layers_;
@@ -107,6 +152,8 @@ class StackModel : public ModelBase {
   void* embed_ = nullptr;
   void* head_ = nullptr;
   float* final_norm_ = nullptr;
+  float* final_b_ = nullptr;
+  float final_alpha_ = 1.f;
   float* inv_freq_ = nullptr;
   // paged caches of the layers that own one: K [blocks * BS, kv_heads * dim], V [blocks * BS, kv_heads * vdim]
   std::vector<void*> kc_, vc_;
@@ -115,7 +162,7 @@ class StackModel : public ModelBase {
   // activations
   int max_tokens_ = 0, max_seqs_ = 0, logit_rows_cap_ = 0, max_rows_ = 0;
   float *x_ = nullptr, *o_ = nullptr, *z_ = nullptr, *pair_out_ = nullptr, *sh_ = nullptr, *xl_ = nullptr, *logits_ = nullptr;
-  void *h_ = nullptr, *qkv_ = nullptr, *attn_ = nullptr, *act_ = nullptr, *hl_ = nullptr;
+  void *h_ = nullptr, *qkv_ = nullptr, *attn_ = nullptr, *act_ = nullptr, *hl_ = nullptr, *qa_ = nullptr;
   int *pair_expert_ = nullptr, *row_token_ = nullptr, *row_pair_ = nullptr, *tile_group_ = nullptr;
   float *pair_weight_ = nullptr, *row_scale_ = nullptr, *gate_ = nullptr;
   bool trace_on_ = false;

@@ -28,7 +28,7 @@ def rms_norm(v, w, eps):
 
 def dyt(x, w, b, alpha):
     """Dynamic Tanh: no statistics of x, an element-wise squash with a learned slope"""
-    return np.tanh(float(alpha) * x) * w + b
+    return np.tanh(float(np.asarray(alpha).reshape(-1)[0]) * x) * w + b
 
 
 def rotary_table(rot, positions):

@@ -80,45 +80,62 @@ def latent_attention(h, tw, p, mx, eps):
     cos, sin = rotary_table(mx["rot"], np.arange(T))
     q_rot = rotate_pairs(q[:, :, dim:], cos, sin)
     k_rot = rotate_pairs(k_rot, cos, sin)
-    sink = tw[p + "sink"]
-    out = np.zeros((T, H, vdim))
-    causal = np.tril(np.ones((T, T), bool))
+    scores = [(q[:, hd, :dim] @ k_un[:, hd].T + q_rot[:, hd] @ k_rot.T) * mx["scale"] for hd in range(H)]
+    return softmax_with_sink(np.stack(scores), v, tw[p + "sink"]).reshape(T, H * vdim) @ tw[p + "o"].T
+
+
+def softmax_with_sink(scores, v, sink, positions=None):
+    """scores [H, Tq, Tk] (already scaled), v [Tk, H, vdim], queries at `positions` (default 0..Tq-1): causal softmax whose denominator
+    also holds exp(sink_h) — a term without key or value -> [Tq, H, vdim]"""
+    H, Tq, Tk = scores.shape
+    p = np.arange(Tq) if positions is None else np.asarray(positions)
+    seen = np.arange(Tk)[None, :] <= p[:, None]
+    out = np.zeros((Tq, H, v.shape[2]))
     for hd in range(H):
-        s = (q[:, hd, :dim] @ k_un[:, hd].T + q_rot[:, hd] @ k_rot.T) * mx["scale"]
-        s = np.where(causal, s, -np.inf)
+        s = np.where(seen, scores[hd], -np.inf)
         m = np.maximum(s.max(-1, keepdims=True), sink[hd])
         e = np.exp(s - m)
         out[:, hd] = (e / (e.sum(-1, keepdims=True) + np.exp(sink[hd] - m))) @ v[:, hd]
-    return out.reshape(T, H * vdim) @ tw[p + "o"].T
+    return out
 
 
-def visible(T, mask):
-    """[T, T] bool: key j is seen from position i"""
-    i, j = np.arange(T)[:, None], np.arange(T)[None, :]
+def visible(T, mask, positions=None):
+    """[Tq, T] bool: key j is seen from position i (queries at `positions`, default 0..T-1)"""
+    i = (np.arange(T) if positions is None else np.asarray(positions))[:, None]
+    j = np.arange(T)[None, :]
     vis = j <= i
     if mask:
-        vis &= (i - j < int(mask["size"])) | (j < int(mask.get("keep_first", 0)))
+        vis = vis & ((i - j < int(mask["size"])) | (j < int(mask.get("keep_first", 0))))
     return vis
 
 
+def sigmoid_weighted_values(q, k, v, scale, mask, head_bias, talk, positions=None):
+    """q [Tq, H, dim] at `positions` over k [Tk, G, dim], v [Tk, G, vdim] at 0..Tk-1: every visible key weighs
+    sigmoid(q . k * scale - slope_h * distance + head_bias_h) (no normalisation over keys), slope_h = 2^(-8 (h + 1) / H); the heads'
+    weights are mixed by `talk`; head h sums the values of its own key/value head -> [Tq, H, vdim]"""
+    Tq, H, _ = q.shape
+    Tk, G, _ = k.shape
+    p = np.arange(Tq) if positions is None else np.asarray(positions)
+    vis = visible(Tk, mask, p)
+    dist = (p[:, None] - np.arange(Tk)[None, :]).astype(np.float64)
+    w = np.zeros((H, Tq, Tk))
+    for hd in range(H):
+        slope = 2.0 ** (-8.0 * (hd + 1) / H)
+        s = (q[:, hd] @ k[:, hd // (H // G)].T) * scale - slope * dist
+        w[hd] = np.where(vis, sigmoid(s + head_bias[hd]), 0.0)
+    w = np.einsum("hg,gij->hij", talk, w)
+    return np.stack([w[hd] @ v[:, hd // (H // G)] for hd in range(H)], 1)
+
+
 def gated_sigmoid_attention(h, tw, p, mx, eps):
-    """biased projections, one RMS norm over all of q and one over all of k, no rotation: a linear distance penalty per head; a window
-    that also keeps the first tokens; every visible key weighs sigmoid(score + head bias), not normalised; the heads' weights are mixed
-    by a matrix; a sigmoid gate on the concatenated heads"""
+    """biased projections, one RMS norm over all of q and one over all of k, no rotation; sigmoid weights in a window that also keeps the
+    first tokens; a sigmoid gate on the concatenated heads"""
     T = h.shape[0]
     H, G, dim, vdim = mx["heads"], mx.get("kv_heads", mx["heads"]), mx["dim"], mx["vdim"]
     q = rms_norm(h @ tw[p + "q"].T + tw[p + "q.b"], tw[p + "q.norm"], eps).reshape(T, H, dim)
     k = rms_norm(h @ tw[p + "k"].T + tw[p + "k.b"], tw[p + "k.norm"], eps).reshape(T, G, dim)
     v = (h @ tw[p + "v"].T + tw[p + "v.b"]).reshape(T, G, vdim)
-    vis = visible(T, mx.get("mask"))
-    dist = (np.arange(T)[:, None] - np.arange(T)[None, :]).astype(np.float64)
-    w = np.zeros((H, T, T))
-    for hd in range(H):
-        slope = 2.0 ** (-8.0 * (hd + 1) / H)
-        s = (q[:, hd] @ k[:, hd // (H // G)].T) * mx["scale"] - slope * dist
-        w[hd] = np.where(vis, sigmoid(s + tw[p + "pb"][hd]), 0.0)
-    w = np.einsum("hg,gij->hij", tw[p + "talk"], w)
-    out = np.stack([w[hd] @ v[:, hd // (H // G)] for hd in range(H)], 1).reshape(T, H * vdim)
+    out = sigmoid_weighted_values(q, k, v, mx["scale"], mx.get("mask"), tw[p + "pb"], tw[p + "talk"]).reshape(T, H * vdim)
     return (out * sigmoid(h @ tw[p + "g"].T)) @ tw[p + "o"].T
 
 

@@ -670,8 +670,8 @@ void vra_stack_op_sigmoid_attention(const void* q, int32_t ldq, void* out, const
                                     const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B,
                                     int32_t T, int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS,
                                     int32_t max_blocks, float scale, int32_t window, int32_t keep_first, const float* slopes,
-                                    const float* head_bias, const float* talk, const float* gate, int32_t gate_ld, int32_t dtype,
-                                    int64_t stream);
+                                    const float* head_bias, const float* talk, const float* gate, int32_t gate_ld, float* scratch,
+                                    int64_t scratch_bytes, int32_t max_len, int32_t dtype, int64_t stream);
 void vra_stack_op_gemm_ex(const void* a, int32_t lda, const void* w, void* out, int32_t ldo, int32_t out_f32, int32_t M, int32_t N,
                           int32_t K, float alpha, const float* bias, int32_t epi, int32_t act, int32_t batch, int64_t a_batch_stride,
                           int64_t w_batch_stride, int64_t out_batch_stride, int32_t dtype, int64_t stream);

@@ -292,27 +292,30 @@ def test_sink_and_planted_latent_key(dt, decode):
                     assert np.abs(got[i]).max() < 0.6, (j, p, kind)
 
 
-def run_sigmoid_attention(L, q, positions, k, v, scale, mask, pb, talk, gate, dt, decode, r, BS=64):
+def run_sigmoid_attention(L, q, positions, k, v, scale, mask, pb, talk, gate, dt, decode, r, BS=64, scratch=True):
     Tq, H, dim = q.shape
     G, vdim = v.shape[1], v.shape[2]
     kc, vc, table = paged(k, v, BS, r, dt)
     slopes = np.array([2.0 ** (-8.0 * (h + 1) / H) for h in range(H)], np.float32)
     win, keep_first = (int(mask["size"]), int(mask.get("keep_first", 0))) if mask else (0, 0)
     args = (H, G, dim, vdim, BS, len(table), scale, win, keep_first, f32(slopes).ptr, f32(pb).ptr, f32(talk).ptr)
+    # scratch for the two-launch forms (the kernels' own one-launch form runs without: scratch=False)
+    nbytes = max(Tq * H * G * vdim, 64 * H * vdim) * 4
+    sc = (empty(nbytes).ptr, nbytes, k.shape[0]) if scratch else (None, 0, 0)
     if decode:
         res = []
         for i in range(Tq):
             o1 = empty(H * vdim * 4)
             L.vra_stack_op_sigmoid_attention(to_dev(q[i].reshape(1, -1), dt).ptr, H * dim, o1.ptr, kc.ptr, vc.ptr, raw([positions[i]], np.int64).ptr,
                                              raw(table, np.uint32).ptr, raw([positions[i] + 1], np.uint32).ptr, None, 1, 1, 1, *args,
-                                             f32(gate[i]).ptr if gate is not None else None, H * vdim, dt, 0)
+                                             f32(gate[i]).ptr if gate is not None else None, H * vdim, *sc, dt, 0)
             check()
             res.append(from_dev(o1, (H, vdim), dt))
         return np.stack(res)
     out = empty(Tq * H * vdim * 4)
     L.vra_stack_op_sigmoid_attention(to_dev(q.reshape(Tq, -1), dt).ptr, H * dim, out.ptr, kc.ptr, vc.ptr, raw(positions, np.int64).ptr, raw(table, np.uint32).ptr,
                                      raw([k.shape[0]], np.uint32).ptr, raw([0, Tq], np.uint32).ptr, 1, Tq, Tq, *args,
-                                     f32(gate).ptr if gate is not None else None, H * vdim, dt, 0)
+                                     f32(gate).ptr if gate is not None else None, H * vdim, *sc, dt, 0)
     check()
     return from_dev(out, (Tq, H, vdim), dt)
 
@@ -320,7 +323,8 @@ def run_sigmoid_attention(L, q, positions, k, v, scale, mask, pb, talk, gate, dt
 @pytest.mark.parametrize("dt", [F32, BF16])
 @pytest.mark.parametrize("decode", [False, True])
 @pytest.mark.parametrize("H,G,dim,vdim,mask", [(6, 3, 16, 24, dict(size=40, keep_first=5)), (4, 4, 8, 8, dict(size=70, keep_first=0)), (2, 1, 5, 7, dict(size=3, keep_first=2)),
-                                               (8, 2, 64, 64, None), (3, 3, 40, 100, dict(size=64, keep_first=64)), (16, 4, 32, 96, dict(size=1, keep_first=1))])
+                                               (8, 2, 64, 64, None), (3, 3, 40, 100, dict(size=64, keep_first=64)), (16, 4, 32, 96, dict(size=1, keep_first=1)),
+                                               (4, 1, 128, 128, dict(size=33, keep_first=40)), (4, 4, 72, 80, dict(size=100, keep_first=3))])
 def test_sigmoid_attention_random(dt, decode, H, G, dim, vdim, mask):
     L = _lib.load()
     r = np.random.default_rng(H * 100 + dim)
@@ -333,10 +337,11 @@ def test_sigmoid_attention_random(dt, decode, H, G, dim, vdim, mask):
     talk = (np.eye(H) + 0.3 * r.standard_normal((H, H))).astype(np.float32)
     gate = r.standard_normal((Tq, H * vdim)).astype(np.float32)
     scale = 1.5 / math.sqrt(dim)
-    got = run_sigmoid_attention(L, q, positions, k, v, scale, mask, pb, talk, gate, dt, decode, r)
     ref = go.sigmoid_weighted_values(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), scale, mask, pb, talk, positions)
     ref = ref * go.sigmoid(gate.astype(np.float64)).reshape(Tq, H, vdim)
-    assert rel(got, ref) < (3e-6 if dt == F32 else 5e-3)
+    for scratch in (True, False):  # the two-launch forms (matrix cores for bf16 prompts, key tiles over workgroups for single tokens) and the plain one
+        got = run_sigmoid_attention(L, q, positions, k, v, scale, mask, pb, talk, gate, dt, decode, r, scratch=scratch)
+        assert rel(got, ref) < (3e-6 if dt == F32 else 5e-3), scratch
 
 
 @pytest.mark.parametrize("dt", [F32, BF16])

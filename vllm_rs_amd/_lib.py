@@ -212,7 +212,7 @@ def load():
     _sig(lib, "vra_stack_op_rope_heads", None, P, c_i32, c_i32, c_i32, P, c_i32, c_i32, c_i32, c_i32, c_i32, P, P, P, c_i32, c_f32, c_i32, c_i32, c_i64)
     _sig(lib, "vra_stack_op_qk_norm_store", None, P, c_i32, c_i32, c_i32, c_i32, P, P, c_f32, P, P, P, P, c_i32, c_i32, c_i64)
     _sig(lib, "vra_stack_op_sigmoid_attention", None, P, c_i32, P, P, P, P, P, P, P, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
-         c_f32, c_i32, c_i32, P, P, P, P, c_i32, c_i32, c_i64)
+         c_f32, c_i32, c_i32, P, P, P, P, c_i32, P, c_i64, c_i32, c_i32, c_i64)
     _sig(lib, "vra_stack_op_gemm_ex", None, P, c_i32, P, P, c_i32, c_i32, c_i32, c_i32, c_i32, c_f32, P, c_i32, c_i32, c_i32, c_i64, c_i64, c_i64, c_i32, c_i64)
     _sig(lib, "vra_stack_op_attention_ex", None, P, c_i32, P, P, P, P, P, P, P, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32, c_i32,
          c_f32, P, c_i32, c_i32, c_i32, c_i64)

@@ -178,5 +178,11 @@ struct StkSigAttnArgs {
   const float* talk = nullptr;       // [H, H]
   const float* gate = nullptr;       // f32 [T, gate_ld], H * vdim columns used
   int gate_ld = 0;
+  // f32 scratch for the forms that sum in two launches (null: the one-launch kernel, any shape).  Prompt portions of bf16 models on the
+  // matrix cores need T * H * G * vdim floats, one token per sequence needs B * S * H * vdim with S <= 64 key tiles; max_len bounds the
+  // context of an unwindowed layer (it fixes S, and with it the order of the sums).
+  float* scratch = nullptr;
+  size_t scratch_bytes = 0;
+  int max_len = 0;
 };
 void vra_stack_sigmoid_attention(const StkSigAttnArgs& a, int dtype, int64_t stream);

@@ -252,6 +252,343 @@ __global__ __launch_bounds__(256) void stk_sig_attn_kernel(StkSigAttnArgs a, int
   }
 }
 
+
+// ------------------------------------------------------------------------------------------------ the same on the matrix cores (bf16)
+// The mixing of the heads is linear in the weights, so it commutes with the sum over keys:
+//   out_h = sum_g talk[h, g] U[g, kv(h)],   U[g, kappa](i) = sum_j w_g(i, j) v_kappa(j).
+// A workgroup of 4 waves owns 64 query rows of ONE head g and GC key/value heads: S^T = K . Q^T on MFMA (K fragments straight from the
+// cache, one tile ahead), the sigmoid weights in f32 per lane, then U^T += V_kappa^T . W^T for each of its value heads with the weights
+// split into a bf16 head and tail (w = hi + lo to 2^-17: f32 weights in effect).  Heads never meet inside the kernel; a second, element-wise
+// launch mixes U and applies the gate.  32-key tiles aligned to absolute positions, ascending; tiles between the kept first tokens and the
+// window are skipped.
+template <int DC, int VT, int GC>
+__global__ __launch_bounds__(256) void stk_sig_prefill_mfma_kernel(StkSigAttnArgs a, float* U) {
+  constexpr int KT = 32, VLD = KT + 8;
+  __shared__ __attribute__((aligned(16))) uint16_t vt[GC * VT * 16 * VLD];
+  const int dim = a.dim, vdim = a.vdim, G = a.G;
+  const int n_gc = (G + GC - 1) / GC;
+  const int b = blockIdx.y, h = blockIdx.z / n_gc, kap0 = (blockIdx.z % n_gc) * GC, gk = h / (a.H / G);
+  const int q0 = a.cu_q[b], q1 = a.cu_q[b + 1];
+  const int t0 = q0 + ((int)gridDim.x - 1 - (int)blockIdx.x) * 64;
+  if (t0 >= q1) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rq = lane & 15, oct = lane >> 4;
+  const int tq = t0 + wave * 16 + rq;
+  const bool qv = tq < q1;
+  const int64_t pq = qv ? a.positions[tq] : -1;
+  const uint16_t* q = (const uint16_t*)a.q;
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  u32x4 qf[DC];
+  for (int c = 0; c < DC; c++) {
+    const int ch = c * 32 + oct * 8;
+    const bool ok = qv && ch < dim;
+    const u32x4 v = *(const u32x4*)(q + (size_t)(ok ? tq : q0) * a.ldq + h * dim + (ok ? ch : 0));
+    qf[c] = ok ? v : zero4;
+  }
+  // the smallest and largest position of the wave's and of the workgroup's rows bound what they can see
+  long long lo = qv ? pq : 0x7fffffffffffffffll, hi = pq;
+  for (int o = 32; o > 0; o >>= 1) lo = min(lo, __shfl_xor(lo, o, 64)), hi = max(hi, __shfl_xor(hi, o, 64));
+  __shared__ long long wlo[4], whi[4];
+  if (lane == 0) wlo[wave] = lo, whi[wave] = hi;
+  __syncthreads();
+  const bool wave_has = hi >= 0;
+  const int64_t wmin = lo, wmax = hi;
+  const int64_t pmin = min(min(wlo[0], wlo[1]), min(wlo[2], wlo[3])), pmax = max(max(whi[0], whi[1]), max(whi[2], whi[3]));
+  const int n_keys = (int)min((int64_t)a.context_lens[b], pmax + 1);
+  const int win = a.window;
+  const int keep_end = win > 0 ? (max(a.keep_first, 0) + KT - 1) / KT * KT : 0;
+  const int win_first = win > 0 ? (int)(max((int64_t)0, pmin - win + 1) / KT) * KT : 0;
+  const int wave_first = win > 0 ? (int)(max((int64_t)0, wmin - win + 1) / KT) * KT : 0;
+  auto next_tile = [&](int kt0) {  // the tile after kt0 that some row of the workgroup may see
+    int n = kt0 + KT;
+    if (win > 0 && n >= keep_end && n < win_first) n = win_first;
+    return n;
+  };
+  const uint16_t* kc = (const uint16_t*)a.kc;
+  const uint16_t* vc = (const uint16_t*)a.vc;
+  const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
+  const int kdim = G * dim, vd_all = G * vdim;
+  f32x4 acc[GC][VT];
+#pragma unroll
+  for (int e = 0; e < GC; e++)
+#pragma unroll
+    for (int t = 0; t < VT; t++) acc[e][t] = vra_zero_acc();
+  const float slope = a.slopes ? a.slopes[h] : 0.f, hb = a.head_bias ? a.head_bias[h] : 0.f;
+  // V item = (value head, pair of neighbouring keys, 8 channels): NV per thread, two 16-byte requests each
+  constexpr int ITEMS = GC * (KT / 2) * VT * 2, NV = (ITEMS + 255) / 256;
+  u32x4 kfn[2][DC], vgn[NV][2];
+  auto page_slot = [&](int kt0) -> int64_t {  // first cache slot of the tile (a 32-key tile lies in one page: the page size is a multiple of 32)
+    const int t = __builtin_amdgcn_readfirstlane(kt0);
+    return t < n_keys ? (int64_t)bt[t / a.BS] * a.BS + t % a.BS : 0;
+  };
+  auto request_tile = [&](int kt0, int64_t slot0) {
+    for (int u = 0; u < 2; u++) {
+      const int key = kt0 + u * 16 + rq;
+      const bool kv = key < n_keys;
+      const uint16_t* kr = kc + (kv ? slot0 + (key - kt0) : 0) * kdim + gk * dim;
+      for (int c = 0; c < DC; c++) {
+        const int ch = c * 32 + oct * 8;
+        const bool ok = kv && ch < dim;
+        const u32x4 kf = *(const u32x4*)(kr + (ok ? ch : 0));
+        kfn[u][c] = ok ? kf : zero4;
+      }
+    }
+    for (int n = 0; n < NV; n++) {
+      const int i = tid + n * 256;
+      const int e = i / ((KT / 2) * VT * 2), r = i % ((KT / 2) * VT * 2);
+      const int kp = r / (VT * 2), c8 = (r % (VT * 2)) * 8;
+      for (int w2 = 0; w2 < 2; w2++) {
+        const int key = kt0 + kp * 2 + w2;
+        const bool ok = i < ITEMS && kap0 + e < G && key < n_keys && c8 < vdim;
+        const u32x4 v = *(const u32x4*)(vc + (ok ? slot0 + (key - kt0) : 0) * vd_all + (ok ? (kap0 + e) * vdim + c8 : 0));
+        vgn[n][w2] = ok ? v : zero4;
+      }
+    }
+  };
+  int kt0 = (win > 0 && keep_end == 0 && win_first > 0) ? win_first : 0;
+  if (kt0 < n_keys) request_tile(kt0, page_slot(kt0));
+  while (kt0 < n_keys) {
+    const int ktn = next_tile(kt0);
+    const int64_t slot_next = page_slot(ktn);
+    u32x4 kfc[2][DC], vgc[NV][2];
+    for (int u = 0; u < 2; u++)
+      for (int c = 0; c < DC; c++) kfc[u][c] = kfn[u][c];
+    for (int n = 0; n < NV; n++) vgc[n][0] = vgn[n][0], vgc[n][1] = vgn[n][1];
+    __syncthreads();
+    for (int n = 0; n < NV; n++) {
+      const int i = tid + n * 256;
+      if (i >= ITEMS) break;
+      const int e = i / ((KT / 2) * VT * 2), r = i % ((KT / 2) * VT * 2);
+      const int kl = (r / (VT * 2)) * 2, c8 = (r % (VT * 2)) * 8;
+      const int pos = ((kl & 15) >> 2) * 8 + (kl >> 4) * 4 + (kl & 3);  // the order in which the lanes hold their weights
+      uint32_t* row = (uint32_t*)(vt + e * VT * 16 * VLD);
+      for (int x = 0; x < 4; x++) {
+        const uint32_t lo0 = vgc[n][0][x] & 0xffffu, hi0 = vgc[n][0][x] >> 16, lo1 = vgc[n][1][x] & 0xffffu, hi1 = vgc[n][1][x] >> 16;
+        row[((c8 + 2 * x) * VLD + pos) >> 1] = lo0 | (lo1 << 16);
+        row[((c8 + 2 * x + 1) * VLD + pos) >> 1] = hi0 | (hi1 << 16);
+      }
+    }
+    __syncthreads();
+    if (ktn < n_keys) request_tile(ktn, slot_next);
+    const int kt = kt0;
+    kt0 = ktn;
+    // (wave-uniform) nothing of this tile is visible to the wave's rows: behind its last row, or before its window and not kept
+    if (!wave_has || kt > wmax || (win > 0 && kt >= keep_end && kt + KT <= wave_first)) continue;
+    f32x4 s[2];
+    s[0] = vra_zero_acc();
+    s[1] = vra_zero_acc();
+    for (int c = 0; c < DC; c++) {
+      BF16::mfma(s[0], __builtin_bit_cast(s16x8, kfc[0][c]), __builtin_bit_cast(s16x8, qf[c]));
+      BF16::mfma(s[1], __builtin_bit_cast(s16x8, kfc[1][c]), __builtin_bit_cast(s16x8, qf[c]));
+    }
+    VRA_MFMA_DRAIN();
+    float pv[8];
+    for (int u = 0; u < 2; u++)
+      for (int j = 0; j < 4; j++) {
+        const int key = kt + u * 16 + oct * 4 + j;
+        const int64_t dist = pq - key;
+        const bool seen = dist >= 0 && key < n_keys && (win <= 0 || dist < win || key < a.keep_first);
+        const float x = s[u][j] * a.scale - slope * (float)dist + hb;
+        pv[u * 4 + j] = seen ? 1.f / (1.f + __expf(-x)) : 0.f;
+      }
+    u32x4 phi, plo;
+    for (int e = 0; e < 4; e++) {
+      const float a0 = pv[2 * e], a1 = pv[2 * e + 1];
+      const uint32_t hi = BF16::pack2(a0, a1);
+      phi[e] = hi;
+      plo[e] = BF16::pack2(a0 - __uint_as_float(hi << 16), a1 - __uint_as_float(hi & 0xffff0000u));
+    }
+#pragma unroll
+    for (int e = 0; e < GC; e++) {
+      u32x4 vf[VT];
+#pragma unroll
+      for (int t = 0; t < VT; t++) vf[t] = *(const u32x4*)(vt + ((e * VT + t) * 16 + rq) * VLD + oct * 8);
+#pragma unroll
+      for (int t = 0; t < VT; t++) BF16::mfma(acc[e][t], __builtin_bit_cast(s16x8, vf[t]), __builtin_bit_cast(s16x8, phi));
+#pragma unroll
+      for (int t = 0; t < VT; t++) BF16::mfma(acc[e][t], __builtin_bit_cast(s16x8, vf[t]), __builtin_bit_cast(s16x8, plo));
+    }
+    VRA_MFMA_DRAIN();
+  }
+  if (!qv) return;
+#pragma unroll
+  for (int e = 0; e < GC; e++) {
+    if (kap0 + e >= G) break;
+    float* out = U + (((size_t)tq * a.H + h) * G + kap0 + e) * vdim;
+#pragma unroll
+    for (int t = 0; t < VT; t++)
+      for (int j = 0; j < 4; j++) {
+        const int c = t * 16 + oct * 4 + j;
+        if (c < vdim) out[c] = acc[e][t][j];
+      }
+  }
+}
+
+// out[t, h, d] = sigmoid(gate[t, h, d]) * sum_g talk[h, g] U[t, g, kv(h), d]   (g ascending)
+template <typename T>
+__global__ __launch_bounds__(256) void stk_sig_mix_kernel(const float* U, const float* talk, const float* gate, int gate_ld, T* out, int H, int G, int vdim) {
+  const int t = blockIdx.x, HV = H * vdim, HG = H / G;
+  for (int c = threadIdx.x; c < HV; c += 256) {
+    const int h = c / vdim, d = c % vdim, kap = h / HG;
+    float s = 0.f;
+    for (int g = 0; g < H; g++) s = fmaf(talk[h * H + g], U[(((size_t)t * H + g) * G + kap) * vdim + d], s);
+    if (gate) s *= sigmoidf_(gate[(size_t)t * gate_ld + c]);
+    El<T>::st(out + (size_t)t * HV + c, s);
+  }
+}
+
+// ------------------------------------------------------------------------------------------------ one token per sequence
+// The keys a token sees (its window and the kept first tokens) are cut into 64-key tiles aligned to absolute positions; workgroup (b, s)
+// takes the tiles s, s + S, ... of sequence b, ALL heads: scores lane-per-key straight from the cache (a key row is read once for the
+// query heads of its group), weights and their mix through LDS, the value product with 8 channels per thread.  Nothing is normalised
+// over keys, so the workgroups' partial sums simply add: a second launch adds them in order s = 0 .. S-1 and applies the gate.
+struct SigTiles {
+  int n_keep, win_first, n;  // tiles [0, n_keep) and [win_first, ...): n in all
+};
+__device__ __forceinline__ SigTiles sig_tiles(int64_t p, int n_keys, int window, int keep_first, int KT) {
+  SigTiles t;
+  const int last = (n_keys - 1) / KT;
+  if (window <= 0) {
+    t.n_keep = 0, t.win_first = 0, t.n = last + 1;
+  } else {
+    t.win_first = (int)(max((int64_t)0, p - window + 1) / KT);
+    t.n_keep = min((max(keep_first, 0) + KT - 1) / KT, t.win_first);
+    t.n = t.n_keep + last - t.win_first + 1;
+  }
+  return t;
+}
+template <typename T>
+__global__ __launch_bounds__(256) void stk_sig_decode_kernel(StkSigAttnArgs a, float* partial, int S) {
+  extern __shared__ float lds[];
+  constexpr int KT = 64;
+  const int dim = a.dim, vdim = a.vdim, H = a.H, G = a.G, HG = H / G, HV = H * vdim, GV = G * vdim;
+  float* qs = lds;                 // [H][dim]
+  float* ws = qs + H * dim;        // [H][64]
+  float* ms = ws + H * KT;         // [H][64]
+  float* tk = ms + H * KT;         // [H][H]
+  int* sl = (int*)(tk + H * H);    // [64] cache slots of the tile's keys
+  const int b = blockIdx.x, sp = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t p = a.positions[b];
+  const int n_keys = (int)min((int64_t)a.context_lens[b], p + 1);
+  const T* q = (const T*)a.q + (size_t)b * a.ldq;
+  for (int i = tid; i < H * dim; i += 256) qs[i] = El<T>::ld(q + i);
+  for (int i = tid; i < H * H; i += 256) tk[i] = a.talk ? a.talk[i] : ((i / H == i % H) ? 1.f : 0.f);
+  const T* kc = (const T*)a.kc;
+  const T* vc = (const T*)a.vc;
+  const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
+  const bool vec = sizeof(T) == 2 && vdim % 8 == 0 && ((uintptr_t)vc % 16) == 0;
+  float acc[16];
+#pragma unroll
+  for (int i = 0; i < 16; i++) acc[i] = 0.f;
+  const SigTiles tl = sig_tiles(p, max(n_keys, 1), a.window, a.keep_first, KT);
+  for (int ti = sp; ti < tl.n && n_keys > 0; ti += S) {
+    const int kt0 = (ti < tl.n_keep ? ti : tl.win_first + ti - tl.n_keep) * KT;
+    __syncthreads();
+    if (tid < KT) {
+      const int key = kt0 + tid;
+      sl[tid] = key < n_keys ? (int)((int64_t)bt[key / a.BS] * a.BS + key % a.BS) : 0;
+    }
+    __syncthreads();
+    {
+      const int key = kt0 + lane;
+      const int64_t dist = p - key;
+      const bool seen = key < n_keys && dist >= 0 && (a.window <= 0 || dist < a.window || key < a.keep_first);
+      for (int g = wave; g < G; g += 4) {
+        const T* kr = kc + (int64_t)sl[lane] * (G * dim) + g * dim;
+        for (int h0 = 0; h0 < HG; h0 += 4) {  // up to four query heads of the group share one pass over the key row
+          float d4[4] = {0.f, 0.f, 0.f, 0.f};
+          const float* q4 = qs + (g * HG + h0) * dim;
+          const int nh = min(4, HG - h0);
+          if (seen) {
+            if (sizeof(T) == 2 && dim % 8 == 0 && ((uintptr_t)kr % 16) == 0) {
+              for (int d = 0; d < dim; d += 8) {
+                const u32x4 v = *(const u32x4*)((const uint16_t*)kr + d);
+                for (int e = 0; e < 4; e++) {
+                  const float k0 = __uint_as_float(v[e] << 16), k1 = __uint_as_float(v[e] & 0xffff0000u);
+                  for (int u = 0; u < 4; u++)
+                    if (u < nh) d4[u] = fmaf(q4[u * dim + d + 2 * e + 1], k1, fmaf(q4[u * dim + d + 2 * e], k0, d4[u]));
+                }
+              }
+            } else {
+              for (int d = 0; d < dim; d++) {
+                const float kv = El<T>::ld(kr + d);
+                for (int u = 0; u < 4; u++)
+                  if (u < nh) d4[u] = fmaf(q4[u * dim + d], kv, d4[u]);
+              }
+            }
+          }
+          for (int u = 0; u < nh; u++) {
+            const int h = g * HG + h0 + u;
+            const float x = d4[u] * a.scale - (a.slopes ? a.slopes[h] : 0.f) * (float)dist + (a.head_bias ? a.head_bias[h] : 0.f);
+            ws[h * KT + lane] = seen ? sigmoidf_(x) : 0.f;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    for (int i = tid; i < H * KT; i += 256) {
+      const int h = i / KT, j = i % KT;
+      float s = 0.f;
+      for (int g = 0; g < H; g++) s = fmaf(tk[h * H + g], ws[g * KT + j], s);
+      ms[i] = s;
+    }
+    __syncthreads();
+    const int nj = min(KT, n_keys - kt0);
+    if (vec) {  // thread = 8 consecutive channels of one head per round: one 16-byte load per key
+#pragma unroll
+      for (int n = 0; n < 2; n++) {
+        const int c8 = (tid + n * 256) * 8;
+        if (c8 < HV) {
+          const int h = c8 / vdim, d = c8 % vdim, g = h / HG;
+          const float* mw = ms + h * KT;
+          for (int j = 0; j < nj; j++) {
+            const u32x4 v = *(const u32x4*)((const uint16_t*)vc + (int64_t)sl[j] * GV + g * vdim + d);
+            const float w = mw[j];
+            for (int e = 0; e < 4; e++) {
+              acc[n * 8 + 2 * e] = fmaf(w, __uint_as_float(v[e] << 16), acc[n * 8 + 2 * e]);
+              acc[n * 8 + 2 * e + 1] = fmaf(w, __uint_as_float(v[e] & 0xffff0000u), acc[n * 8 + 2 * e + 1]);
+            }
+          }
+        }
+      }
+    } else {
+#pragma unroll
+      for (int n = 0; n < 16; n++) {
+        const int c = tid + n * 256;
+        if (c < HV) {
+          const int h = c / vdim, d = c % vdim, g = h / HG;
+          const float* mw = ms + h * KT;
+          float o = acc[n];
+          for (int j = 0; j < nj; j++) o = fmaf(mw[j], El<T>::ld(vc + (int64_t)sl[j] * GV + g * vdim + d), o);
+          acc[n] = o;
+        }
+      }
+    }
+  }
+  float* po = partial + ((size_t)b * S + sp) * HV;
+  if (vec) {
+    for (int n = 0; n < 2; n++) {
+      const int c8 = (tid + n * 256) * 8;
+      if (c8 < HV)
+        for (int e = 0; e < 8; e++) po[c8 + e] = acc[n * 8 + e];
+    }
+  } else {
+    for (int n = 0; n < 16; n++) {
+      const int c = tid + n * 256;
+      if (c < HV) po[c] = acc[n];
+    }
+  }
+}
+template <typename T>
+__global__ __launch_bounds__(256) void stk_sig_decode_sum_kernel(const float* partial, int S, const float* gate, int gate_ld, T* out, int HV) {
+  const int b = blockIdx.x;
+  for (int c = threadIdx.x; c < HV; c += 256) {
+    float s = 0.f;
+    for (int i = 0; i < S; i++) s += partial[((size_t)b * S + i) * HV + c];
+    if (gate) s *= sigmoidf_(gate[(size_t)b * gate_ld + c]);
+    El<T>::st(out + (size_t)b * HV + c, s);
+  }
+}
+
 }  // namespace
 
 // ================================================================================================ launchers
@@ -308,6 +645,42 @@ void vra_stack_sigmoid_attention(const StkSigAttnArgs& a, int dtype, int64_t str
   hipStream_t st = as_stream(stream);
   const int HV = a.H * a.vdim;
   const bool decode = !a.cu_q;
+  if (decode && a.scratch && HV <= 4096) {
+    // tiles a token can see: the kept first tokens, its window and one more for the window's alignment; without a window, the context
+    int S = a.window > 0 ? (std::max(a.keep_first, 0) + 63) / 64 + (a.window + 63) / 64 + 1 : std::max(1, (std::max(a.max_len, 1) + 63) / 64);
+    S = std::min(S, 64);
+    const size_t lds = ((size_t)a.H * a.dim + 2 * (size_t)a.H * 64 + (size_t)a.H * a.H + 64) * sizeof(float);
+    if (lds <= 64 * 1024 && (size_t)a.B * S * HV * sizeof(float) <= a.scratch_bytes) {
+      dim3 grid(a.B, S);
+      if (dtype == VRA_F32) {
+        launch_checked("stack sigmoid attention (decode)", [&] { stk_sig_decode_kernel<float><<<grid, 256, lds, st>>>(a, a.scratch, S); });
+        launch_checked("stack sigmoid attention (decode sum)", [&] { stk_sig_decode_sum_kernel<float><<<a.B, 256, 0, st>>>(a.scratch, S, a.gate, a.gate_ld, (float*)a.out, HV); });
+      } else {
+        launch_checked("stack sigmoid attention (decode)", [&] { stk_sig_decode_kernel<uint16_t><<<grid, 256, lds, st>>>(a, a.scratch, S); });
+        launch_checked("stack sigmoid attention (decode sum)", [&] { stk_sig_decode_sum_kernel<uint16_t><<<a.B, 256, 0, st>>>(a.scratch, S, a.gate, a.gate_ld, (uint16_t*)a.out, HV); });
+      }
+      return;
+    }
+  }
+  if (!decode && dtype == VRA_BF16 && a.scratch && a.talk && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 128 && a.vdim <= 128 && a.ldq % 8 == 0 &&
+      ((uintptr_t)a.q % 16 == 0) && ((uintptr_t)a.kc % 16 == 0) && ((uintptr_t)a.vc % 16 == 0) && a.BS % 32 == 0 &&
+      (size_t)a.T * a.H * a.G * a.vdim * sizeof(float) <= a.scratch_bytes) {
+    const int gc = a.G >= 2 ? 2 : 1;  // value heads per workgroup: two keep the accumulators in registers, the scores are computed G / 2 times
+    dim3 grid((a.max_q + 63) / 64, a.B, a.H * ((a.G + gc - 1) / gc));
+#define STK_SGM(DCV, VTV, GCV) launch_checked("stack sigmoid attention (prefill, mfma)", [&] { stk_sig_prefill_mfma_kernel<DCV, VTV, GCV><<<grid, 256, 0, st>>>(a, a.scratch); })
+    if (a.dim <= 64 && a.vdim <= 64) {
+      if (gc == 2) STK_SGM(2, 4, 2);
+      else STK_SGM(2, 4, 1);
+    } else {
+      if (gc == 2) STK_SGM(4, 8, 2);
+      else STK_SGM(4, 8, 1);
+    }
+#undef STK_SGM
+    launch_checked("stack sigmoid attention (mix)", [&] {
+      stk_sig_mix_kernel<uint16_t><<<a.T, 256, 0, st>>>(a.scratch, a.talk, a.gate, a.gate_ld, (uint16_t*)a.out, a.H, a.G, a.vdim);
+    });
+    return;
+  }
   int qt, nacc;
   if (decode) qt = 1, nacc = HV <= 4096 ? 16 : 64;
   else if (HV <= 256) qt = 16, nacc = 16;
@@ -369,12 +742,12 @@ extern "C" void vra_stack_op_sigmoid_attention(const void* q, int32_t ldq, void*
                                                const uint32_t* block_tables, const uint32_t* context_lens, const uint32_t* cu_q, int32_t B, int32_t T,
                                                int32_t max_q, int32_t H, int32_t G, int32_t dim, int32_t vdim, int32_t BS, int32_t max_blocks, float scale,
                                                int32_t window, int32_t keep_first, const float* slopes, const float* head_bias, const float* talk,
-                                               const float* gate, int32_t gate_ld, int32_t dtype, int64_t stream) {
+                                               const float* gate, int32_t gate_ld, float* scratch, int64_t scratch_bytes, int32_t max_len, int32_t dtype, int64_t stream) {
   StkSigAttnArgs a;
   a.q = q, a.ldq = ldq, a.out = out, a.kc = kc, a.vc = vc, a.positions = positions, a.block_tables = block_tables, a.context_lens = context_lens;
   a.cu_q = cu_q, a.B = B, a.T = T, a.max_q = max_q, a.H = H, a.G = G, a.dim = dim, a.vdim = vdim, a.BS = BS, a.max_blocks = max_blocks;
   a.scale = scale, a.window = window, a.keep_first = keep_first, a.slopes = slopes, a.head_bias = head_bias, a.talk = talk, a.gate = gate;
-  a.gate_ld = gate_ld;
+  a.gate_ld = gate_ld, a.scratch = scratch, a.scratch_bytes = (size_t)scratch_bytes, a.max_len = max_len;
   vra_stack_sigmoid_attention(a, dtype, stream);
 }
 // the matrix product with every option of StkGemmArgs: bias, batched form, kind of the gated pair

@@ -552,6 +552,15 @@ bool StackModel::init_buffers(int max_tokens, int max_seqs) {
       !(pair_out_ = (float*)dalloc(T * std::max<size_t>(top, 1) * W * 4)) || !(sh_ = (float*)dalloc(T * W * 4)) || !(xl_ = (float*)dalloc(R * W * 4)) ||
       !(hl_ = dalloc(R * W * es_)) || !(logits_ = (float*)dalloc(R * (size_t)vocab_ * 4)) || !(qa_ = dalloc(std::max<size_t>(T * nqa, 4) * es_)))
     return false;
+  // sigmoid attention sums in two launches: per-head-pair sums of a prompt portion (bf16, at most 1 GiB: longer steps take the one-launch
+  // kernel), per-tile partial sums of decoded tokens
+  for (const StackLayer& L : layers_) {
+    if (L.mixer != 2) continue;
+    const size_t hv = (size_t)L.heads * L.vdim;
+    if (dt_ == VRA_BF16) sig_scratch_bytes_ = std::max(sig_scratch_bytes_, std::min<size_t>(T * hv * L.kv_heads * 4, (size_t)1 << 30));
+    sig_scratch_bytes_ = std::max(sig_scratch_bytes_, (size_t)max_seqs * 64 * hv * 4);
+  }
+  if (sig_scratch_bytes_ && !(sig_scratch_ = (float*)dalloc(sig_scratch_bytes_))) return false;
   const size_t P = T * std::max<size_t>(top, 1);
   if (!(pair_expert_ = (int*)dalloc(P * 4)) || !(pair_weight_ = (float*)dalloc(P * 4)) || !(gate_ = (float*)dalloc(T * 4)) ||
       !(row_token_ = (int*)dalloc((size_t)max_rows_ * 4)) || !(row_pair_ = (int*)dalloc((size_t)max_rows_ * 4)) ||
@@ -725,6 +734,7 @@ bool StackModel::mixer_sigmoid(const StackLayer& L, const InputMetadata& md, int
   a.B = B, a.T = T, a.max_q = md.is_prefill ? md.max_seqlen_q : 1, a.H = L.heads, a.G = L.kv_heads, a.dim = L.dim, a.vdim = L.vdim;
   a.BS = ec_.block_size, a.max_blocks = md.max_blocks, a.scale = L.scale, a.window = L.window, a.keep_first = L.keep_first;
   a.slopes = L.slopes, a.head_bias = L.head_bias, a.talk = L.talk, a.gate = z_ + L.nq() + L.nk() + L.nv(), a.gate_ld = n4;
+  a.scratch = sig_scratch_, a.scratch_bytes = sig_scratch_bytes_, a.max_len = mc_.max_position_embeddings;
   vra_stack_sigmoid_attention(a, dt_, stream);
   StkGemmArgs o;
   o.a = attn_, o.lda = L.heads * L.vdim, o.w = L.o, o.M = T, o.N = W, o.K = L.heads * L.vdim, o.out = o_, o.ldo = W, o.out_f32 = 1;

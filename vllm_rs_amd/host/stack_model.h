@@ -165,6 +165,8 @@ class StackModel : public ModelBase {
   void *h_ = nullptr, *qkv_ = nullptr, *attn_ = nullptr, *act_ = nullptr, *hl_ = nullptr, *qa_ = nullptr;
   int *pair_expert_ = nullptr, *row_token_ = nullptr, *row_pair_ = nullptr, *tile_group_ = nullptr;
   float *pair_weight_ = nullptr, *row_scale_ = nullptr, *gate_ = nullptr;
+  float* sig_scratch_ = nullptr;
+  size_t sig_scratch_bytes_ = 0;
   bool trace_on_ = false;
   float* trace_ = nullptr;
   size_t trace_cap_ = 0, trace_bytes_ = 0;

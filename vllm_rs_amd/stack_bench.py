@@ -1,4 +1,5 @@
-"""Throughput of a layer-stack model (Ditilix design) beside the dense bf16 Llama of the same widths — `python bench.py --design ditilix`.
+"""Throughput of a layer-stack model (Ditilix or Gaperax design) beside the dense bf16 Llama of the same widths —
+`python bench.py --design ditilix|gaperax`.
 
 Random weights of layer sizes that resemble a real model; for each size one JSON line with prefill tokens/s (one prompt of
 `prefill_tokens`, best of three engine steps) and decode tokens/s (batches of 1 and 8 behind 512-token prompts, HIP-event time of
@@ -45,6 +46,33 @@ def stack_costs(cj):
         wbytes += 2 * act
     head = cj["vocab"] * W
     return flops + 2 * head, wbytes + 2 * head
+
+
+def gaperax_config(width, heads, kv_heads, dim, ff, layers, vocab, kv_rank, q_rank, rot_dim, window, keep_first):
+    """config.json dict of a Gaperax model: every fourth layer (from the first) a latent attention, the others windowed sigmoid attention"""
+    lat = dict(heads=heads, dim=dim, rot_dim=rot_dim, vdim=dim, kv_rank=kv_rank, q_rank=q_rank, scale=(dim + rot_dim) ** -0.5,
+               rot=dict(base=5e5, dims=rot_dim, scaling=dict(factor=8.0, original=8192, fast=32.0, slow=1.0)))
+    sig = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=dim, scale=dim ** -0.5, mask=dict(size=window, keep_first=keep_first))
+    ls = [dict(type="latent_attention" if i % 4 == 0 else "attention", mixer=lat if i % 4 == 0 else sig, mlp=dict(kind="dense", ff=ff)) for i in range(layers)]
+    return dict(architecture="Gaperax", width=width, vocab=vocab, norm=dict(eps=1e-6), layers=ls)
+
+
+def gaperax_costs(cj):
+    """(matrix FLOPs per token without attention, weight bytes a one-token step reads) of a Gaperax config"""
+    W, n = cj["width"], 0
+    for layer in cj["layers"]:
+        mx = layer["mixer"]
+        H, dim, vdim = mx["heads"], mx["dim"], mx["vdim"]
+        if layer["type"] == "latent_attention":
+            rd, kr, qr = mx["rot_dim"], mx["kv_rank"], mx["q_rank"]
+            n += W * (qr + kr + rd) + qr * H * (dim + rd) + H * dim * kr + H * kr * vdim + H * vdim * W
+        else:
+            G = mx.get("kv_heads", H)
+            n += W * (H * dim + G * dim + G * vdim + H * vdim) + H * vdim * W
+        if layer.get("mlp"):
+            n += 3 * W * layer["mlp"]["ff"]
+    n += cj["vocab"] * W
+    return 2 * n, 2 * n
 
 
 def llama_costs(cfg):
@@ -96,18 +124,30 @@ SIZES = {
 }
 
 
-def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None):
+GAPERAX_SIZES = {
+    # name: (width, heads, kv_heads, head size, ff, layers, vocab, kv latent, q latent, rotated part, window, kept first tokens)
+    "gaperax-2048": (2048, 16, 4, 128, 8192, 4, 32000, 192, 768, 64, 1024, 16),
+    "gaperax-4096": (4096, 32, 8, 128, 14336, 2, 32000, 192, 1536, 64, 1024, 16),
+}
+
+
+def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None, design="ditilix"):
     from . import _lib, checkpoint
     from .engine import BF16, Engine
     L = _lib.load()
     lines = []
-    for name in (sizes or SIZES):
-        width, heads, kvh, dim, ff, layers, vocab, experts, top, eff, sff, share = SIZES[name]
-        cj = stack_config(width, heads, kvh, dim, ff, layers, vocab, experts, top, eff, sff, share)
+    table = GAPERAX_SIZES if design == "gaperax" else SIZES
+    for name in (sizes or table):
+        if design == "gaperax":
+            width, heads, kvh, dim, ff, layers, vocab, kr, qr, rd, window, keep_first = table[name]
+            cj = gaperax_config(width, heads, kvh, dim, ff, layers, vocab, kr, qr, rd, window, keep_first)
+        else:
+            width, heads, kvh, dim, ff, layers, vocab, experts, top, eff, sff, share = table[name]
+            cj = stack_config(width, heads, kvh, dim, ff, layers, vocab, experts, top, eff, sff, share)
         eng = Engine(checkpoint.parse_config(cj), num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
         res = dict(stack=measure(eng, L, vocab, prefill_tokens, steps, warmup))
         eng.close()
-        res["stack"]["flops_per_token"], res["stack"]["weight_bytes_per_step"] = stack_costs(cj)
+        res["stack"]["flops_per_token"], res["stack"]["weight_bytes_per_step"] = gaperax_costs(cj) if design == "gaperax" else stack_costs(cj)
         lcfg = dict(arch="llama", hidden_size=width, intermediate_size=ff, num_layers=layers, num_heads=heads, num_kv_heads=kvh, head_dim=dim,
                     vocab_size=vocab, max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0, quant_method=None, dtype=BF16)
         eng = Engine(lcfg, num_gpu_blocks=512, max_num_seqs=8, max_model_len=4096, use_graph=graph).init_synthetic()
@@ -117,7 +157,7 @@ def main(steps=64, warmup=8, prefill_tokens=2048, graph=True, sizes=None):
         for m in res.values():
             m["prefill_matrix_tflops"] = m["prefill_tokens_per_s"] * m["flops_per_token"] / 1e12
             m["decode_bs1_weight_gb_per_s"] = m["weight_bytes_per_step"] / (m["decode_bs1_ms_per_step"] / 1e3) / 1e9
-        line = dict(metric="stack_vs_dense_llama", size=name, design="Ditilix", dtype="bf16", data="synthetic", prefill_tokens=prefill_tokens,
+        line = dict(metric="stack_vs_dense_llama", size=name, design="Gaperax" if design == "gaperax" else "Ditilix", dtype="bf16", data="synthetic", prefill_tokens=prefill_tokens,
                     decode_context=512, steps=steps, **res)
         print(json.dumps(line), flush=True)
         lines.append(line)

@@ -500,12 +500,17 @@ __global__ __launch_bounds__(256) void stk_sig_decode_kernel(StkSigAttnArgs a, f
           const int nh = min(4, HG - h0);
           if (seen) {
             if (sizeof(T) == 2 && dim % 8 == 0 && ((uintptr_t)kr % 16) == 0) {
-              for (int d = 0; d < dim; d += 8) {
-                const u32x4 v = *(const u32x4*)((const uint16_t*)kr + d);
-                for (int e = 0; e < 4; e++) {
-                  const float k0 = __uint_as_float(v[e] << 16), k1 = __uint_as_float(v[e] & 0xffff0000u);
-                  for (int u = 0; u < 4; u++)
-                    if (u < nh) d4[u] = fmaf(q4[u * dim + d + 2 * e + 1], k1, fmaf(q4[u * dim + d + 2 * e], k0, d4[u]));
+              for (int d0 = 0; d0 < dim; d0 += 32) {  // four 16-byte requests of the key row in flight, then their sums (d ascending)
+                u32x4 kv4[4];
+                for (int x = 0; x < 4; x++) kv4[x] = *(const u32x4*)((const uint16_t*)kr + (d0 + 8 * x < dim ? d0 + 8 * x : 0));
+                for (int x = 0; x < 4; x++) {
+                  const int d = d0 + 8 * x;
+                  if (d >= dim) break;
+                  for (int e = 0; e < 4; e++) {
+                    const float k0 = __uint_as_float(kv4[x][e] << 16), k1 = __uint_as_float(kv4[x][e] & 0xffff0000u);
+                    for (int u = 0; u < 4; u++)
+                      if (u < nh) d4[u] = fmaf(q4[u * dim + d + 2 * e + 1], k1, fmaf(q4[u * dim + d + 2 * e], k0, d4[u]));
+                  }
                 }
               }
             } else {
@@ -540,13 +545,19 @@ __global__ __launch_bounds__(256) void stk_sig_decode_kernel(StkSigAttnArgs a, f
         if (c8 < HV) {
           const int h = c8 / vdim, d = c8 % vdim, g = h / HG;
           const float* mw = ms + h * KT;
-          for (int j = 0; j < nj; j++) {
-            const u32x4 v = *(const u32x4*)((const uint16_t*)vc + (int64_t)sl[j] * GV + g * vdim + d);
-            const float w = mw[j];
-            for (int e = 0; e < 4; e++) {
-              acc[n * 8 + 2 * e] = fmaf(w, __uint_as_float(v[e] << 16), acc[n * 8 + 2 * e]);
-              acc[n * 8 + 2 * e + 1] = fmaf(w, __uint_as_float(v[e] & 0xffff0000u), acc[n * 8 + 2 * e + 1]);
+          for (int j0 = 0; j0 < nj; j0 += 8) {  // eight value rows requested together; rows beyond the tile count with weight 0
+            u32x4 v[8];
+            float w[8];
+            for (int u = 0; u < 8; u++) {
+              const bool in = j0 + u < nj;
+              v[u] = *(const u32x4*)((const uint16_t*)vc + (int64_t)sl[in ? j0 + u : j0] * GV + g * vdim + d);
+              w[u] = in ? mw[j0 + u] : 0.f;
             }
+            for (int u = 0; u < 8; u++)
+              for (int e = 0; e < 4; e++) {
+                acc[n * 8 + 2 * e] = fmaf(w[u], __uint_as_float(v[u][e] << 16), acc[n * 8 + 2 * e]);
+                acc[n * 8 + 2 * e + 1] = fmaf(w[u], __uint_as_float(v[u][e] & 0xffff0000u), acc[n * 8 + 2 * e + 1]);
+              }
           }
         }
       }
@@ -580,13 +591,19 @@ __global__ __launch_bounds__(256) void stk_sig_decode_kernel(StkSigAttnArgs a, f
 }
 template <typename T>
 __global__ __launch_bounds__(256) void stk_sig_decode_sum_kernel(const float* partial, int S, const float* gate, int gate_ld, T* out, int HV) {
-  const int b = blockIdx.x;
-  for (int c = threadIdx.x; c < HV; c += 256) {
-    float s = 0.f;
-    for (int i = 0; i < S; i++) s += partial[((size_t)b * S + i) * HV + c];
-    if (gate) s *= sigmoidf_(gate[(size_t)b * gate_ld + c]);
-    El<T>::st(out + (size_t)b * HV + c, s);
+  const int b = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+  if (c >= HV) return;
+  const float* pp = partial + (size_t)b * S * HV + c;
+  float s = 0.f;
+  int i = 0;
+  for (; i + 8 <= S; i += 8) {  // (eight requests in flight; the sum keeps the order i = 0 .. S-1)
+    float v[8];
+    for (int u = 0; u < 8; u++) v[u] = pp[(size_t)(i + u) * HV];
+    for (int u = 0; u < 8; u++) s += v[u];
   }
+  for (; i < S; i++) s += pp[(size_t)i * HV];
+  if (gate) s *= sigmoidf_(gate[(size_t)b * gate_ld + c]);
+  El<T>::st(out + (size_t)b * HV + c, s);
 }
 
 }  // namespace
@@ -654,10 +671,10 @@ void vra_stack_sigmoid_attention(const StkSigAttnArgs& a, int dtype, int64_t str
       dim3 grid(a.B, S);
       if (dtype == VRA_F32) {
         launch_checked("stack sigmoid attention (decode)", [&] { stk_sig_decode_kernel<float><<<grid, 256, lds, st>>>(a, a.scratch, S); });
-        launch_checked("stack sigmoid attention (decode sum)", [&] { stk_sig_decode_sum_kernel<float><<<a.B, 256, 0, st>>>(a.scratch, S, a.gate, a.gate_ld, (float*)a.out, HV); });
+        launch_checked("stack sigmoid attention (decode sum)", [&] { stk_sig_decode_sum_kernel<float><<<dim3(a.B, (HV + 255) / 256), 256, 0, st>>>(a.scratch, S, a.gate, a.gate_ld, (float*)a.out, HV); });
       } else {
         launch_checked("stack sigmoid attention (decode)", [&] { stk_sig_decode_kernel<uint16_t><<<grid, 256, lds, st>>>(a, a.scratch, S); });
-        launch_checked("stack sigmoid attention (decode sum)", [&] { stk_sig_decode_sum_kernel<uint16_t><<<a.B, 256, 0, st>>>(a.scratch, S, a.gate, a.gate_ld, (uint16_t*)a.out, HV); });
+        launch_checked("stack sigmoid attention (decode sum)", [&] { stk_sig_decode_sum_kernel<uint16_t><<<dim3(a.B, (HV + 255) / 256), 256, 0, st>>>(a.scratch, S, a.gate, a.gate_ld, (uint16_t*)a.out, HV); });
       }
       return;
     }

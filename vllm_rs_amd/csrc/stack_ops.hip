@@ -1061,6 +1061,7 @@ void vra_stack_attention(const StkAttnArgs& a, int dtype, int64_t stream) {
 #define STK_PFM(DCV, VTV) launch_checked("stack attention (prefill, mfma)", [&] { stk_attn_prefill_mfma_kernel<DCV, VTV><<<grid, 256, 0, st>>>(a); })
     if (a.dim <= 64 && a.vdim <= 64) STK_PFM(2, 4);
     else if (a.dim <= 128 && a.vdim <= 128) STK_PFM(4, 8);
+    else if (a.vdim <= 192) STK_PFM(8, 12);  // (a latent cache's rows: 192 value channels do not pay for 256)
     else STK_PFM(8, 16);
 #undef STK_PFM
     return;

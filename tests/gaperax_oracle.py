@@ -14,7 +14,7 @@ from tests.stack_oracle import bf16_round  # noqa: F401  (re-exported: the tests
 
 
 def sigmoid(z):
-    return 1.0 / (1.0 + np.exp(-z))
+    return 0.5 * (1.0 + np.tanh(0.5 * np.asarray(z, np.float64)))  # (= 1 / (1 + e^-z), without the overflow of e^-z far below 0)
 
 
 def gelu_tanh(z):

@@ -324,7 +324,8 @@ def run_sigmoid_attention(L, q, positions, k, v, scale, mask, pb, talk, gate, dt
 @pytest.mark.parametrize("decode", [False, True])
 @pytest.mark.parametrize("H,G,dim,vdim,mask", [(6, 3, 16, 24, dict(size=40, keep_first=5)), (4, 4, 8, 8, dict(size=70, keep_first=0)), (2, 1, 5, 7, dict(size=3, keep_first=2)),
                                                (8, 2, 64, 64, None), (3, 3, 40, 100, dict(size=64, keep_first=64)), (16, 4, 32, 96, dict(size=1, keep_first=1)),
-                                               (4, 1, 128, 128, dict(size=33, keep_first=40)), (4, 4, 72, 80, dict(size=100, keep_first=3))])
+                                               (4, 1, 128, 128, dict(size=33, keep_first=40)), (4, 4, 72, 80, dict(size=100, keep_first=3)),
+                                               (8, 8, 32, 32, dict(size=50, keep_first=2)), (6, 3, 32, 32, dict(size=90, keep_first=0)), (12, 3, 64, 32, None)])
 def test_sigmoid_attention_random(dt, decode, H, G, dim, vdim, mask):
     L = _lib.load()
     r = np.random.default_rng(H * 100 + dim)
@@ -346,13 +347,14 @@ def test_sigmoid_attention_random(dt, decode, H, G, dim, vdim, mask):
 
 @pytest.mark.parametrize("dt", [F32, BF16])
 @pytest.mark.parametrize("decode", [False, True])
-def test_sigmoid_attention_window_edges_and_kept_tokens(dt, decode):
+@pytest.mark.parametrize("H,G,dim,vdim", [(2, 1, 8, 4), (4, 2, 16, 16), (2, 2, 16, 16)])  # (bf16 prompts: FMA kernel, all-heads and per-head matrix-core kernels)
+def test_sigmoid_attention_window_edges_and_kept_tokens(dt, decode, H, G, dim, vdim):
     """Every key weighs about e^-12 except ONE, whose score is made large: the output is its value (a marker) exactly when the design
     lets the query see it — the last key inside the window and the first one outside, the last kept first token and the one after it, at
     page borders, far back, the query's own position and the position before the key arrives."""
     L = _lib.load()
     r = np.random.default_rng(13)
-    Tk, H, G, dim, vdim = 700, 2, 1, 8, 4
+    Tk = 700
     size, keep_first = 150, 12
     mask = dict(size=size, keep_first=keep_first)
     pb, talk = np.full(H, -12.0, np.float32), np.eye(H, dtype=np.float32)
@@ -365,15 +367,16 @@ def test_sigmoid_attention_window_edges_and_kept_tokens(dt, decode):
     cases += [(64, 63, False), (64, 64, True), (63, 64, True), (128, 277, True), (127, 277, False), (5, 5, True), (19, 19, True), (25, 100, True), (25, 175, False)]
     for j, p, seen in cases:
         k, v = base_k.copy(), base_v.copy()
-        k[j, 0] = 16.0 * u
-        v[j, 0] = 5.0
+        k[j, :] = 16.0 * u
+        v[j, :] = 5.0
         q = np.tile(8.0 * u, (1, H, 1)).astype(np.float32)  # score 8 * 16 * 0.25 = 32, minus the distance penalty (at most 700 / 16), plus -12
         positions = np.array([p], np.int64)
-        got = run_sigmoid_attention(L, q, positions, k, v, 0.25, mask, pb, talk, None, dt, decode, r)
+        # (bf16 prompts: with scratch short steps take the per-head matrix-core kernel, without it the all-heads one where the shape allows)
+        got = run_sigmoid_attention(L, q, positions, k, v, 0.25, mask, pb, talk, None, dt, decode, r, scratch=(j + p) % 2 == 0)
         ref = go.sigmoid_weighted_values(q.astype(np.float64), k.astype(np.float64), v.astype(np.float64), 0.25, mask, pb, talk, positions)
         assert np.abs(got - ref).max() < (1e-4 if dt == F32 else 3e-2), (j, p)
-        # head 1 (slope 2^-8) always keeps the planted weight near 1 when the key is seen
-        assert (np.abs(got[0, 1] - 5.0).max() < 0.1) == seen, (j, p, seen, got[0, 1])
+        # the last head (slope 2^-8) always keeps the planted weight near 1 when the key is seen
+        assert (np.abs(got[0, H - 1] - 5.0).max() < 0.1) == seen, (j, p, seen, got[0, H - 1])
         if not seen:
             assert np.abs(got).max() < 0.05, (j, p)
 
@@ -551,6 +554,29 @@ def test_mixed_steps_and_reused_pages(model):
             if live[i] == lens[i]:
                 del live[i]
     agree(np.concatenate(got_rows), np.concatenate(ref_rows), dt)
+
+
+def test_long_prompt_in_one_step_and_in_portions():
+    """a 1700-token prompt: bf16 steps of this size run the sigmoid attention's all-heads kernel, shorter portions the per-head one; both agree
+    with the oracle, and the long step with its portions"""
+    cfg = dict(config_a(), layers=[dict(type="attention", mixer=windowed(heads=8, kv_heads=2, dim=32, vdim=32, size=300, keep_first=7), mlp=dict(kind="dense", ff=64)),
+                                   dict(type="latent_attention", mixer=latent(), mlp=None)])
+    tensors = go.random_tensors(cfg, 23)
+    toks = tokens_of(cfg, 1700, 8)
+    want = list(range(0, 1700, 53)) + [1699]
+    ref = go.forward(cfg, tensors, toks)[want]
+    for dt in (F32, BF16):
+        eng = build(cfg, tensors, dt, blocks=56, max_model_len=1792)
+        whole = eng.replay_step([(1, toks, want)], [1])
+        agree(whole, ref, dt, "whole")
+        parts, at = [], 0
+        for c in (700, 40, 960):
+            parts.append(eng.replay_step([(2, toks[at:at + c], [w - at for w in want if at <= w < at + c])], [2] if at + c == 1700 else []))
+            at += c
+        eng.close()
+        parts = np.concatenate(parts)
+        agree(parts, ref, dt, "portions")
+        assert rel(parts, whole) < (1e-5 if dt == F32 else 3e-2)
 
 
 def test_long_decoding(model):

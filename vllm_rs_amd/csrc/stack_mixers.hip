@@ -385,10 +385,10 @@ __global__ __launch_bounds__(256) void stk_sig_prefill_mfma_kernel(StkSigAttnArg
     for (int u = 0; u < 2; u++)
       for (int j = 0; j < 4; j++) {
         const int key = kt + u * 16 + oct * 4 + j;
-        const int64_t dist = pq - key;
-        const bool seen = dist >= 0 && key < n_keys && (win <= 0 || dist < win || key < a.keep_first);
+        const int dist = (int)pq - key;  // (no short-circuit evaluation: the weights of a tile are straight-line code)
+        const bool seen = (dist >= 0) & (key < n_keys) & ((win <= 0) | (dist < win) | (key < a.keep_first));
         const float x = s[u][j] * a.scale - slope * (float)dist + hb;
-        pv[u * 4 + j] = seen ? 1.f / (1.f + __expf(-x)) : 0.f;
+        pv[u * 4 + j] = seen ? __builtin_amdgcn_rcpf(1.f + __expf(-x)) : 0.f;  // (hardware exponential and reciprocal: no branches)
       }
     u32x4 phi, plo;
     for (int e = 0; e < 4; e++) {
@@ -421,6 +421,194 @@ __global__ __launch_bounds__(256) void stk_sig_prefill_mfma_kernel(StkSigAttnArg
         if (c < vdim) out[c] = acc[e][t][j];
       }
   }
+}
+
+// All heads in one workgroup of NW waves (H = NW HPW; a wave's HPW heads lie in one key/value group): 16 query rows, wave w owns
+// the heads [w HPW, (w + 1) HPW).  (Eight waves of two heads for 16 heads measured slower than four waves of four: 357 against
+// 290 us at 2048 tokens — more waves at the two meetings, every V tile transposed twice.)  Per 32-key tile every wave computes the weights of its own heads on MFMA and leaves them in LDS (f32,
+// in the lanes' own key order), all waves meet, every wave mixes ALL heads' weights into those of its own heads (g ascending), and
+// multiplies them — split hi + lo — with the V tile of its key/value head, which it transposed into its own part of LDS.  One value product
+// per head instead of one per (head, key/value head): the kernel of choice when the shape allows it; it writes the gated output itself.
+template <int DC, int VT, int HPW, int NW>
+__global__ __launch_bounds__(64 * NW) void stk_sig_prefill_heads_kernel(StkSigAttnArgs a) {
+  constexpr int KT = 32, VLD = KT + 8, QR = 16, WLD = KT + 4;  // (WLD: rows of the weight buffer 16 bytes apart in the banks)
+  extern __shared__ __attribute__((aligned(16))) float lds[];
+  const int dim = a.dim, vdim = a.vdim, H = a.H, G = a.G, HG = H / G;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, rq = lane & 15, oct = lane >> 4;
+  float* wbuf = lds;                                   // [H][16 rows][WLD: 32 key places + 4]
+  float* tk = wbuf + H * QR * WLD;                      // [H][H]
+  uint16_t* vt = (uint16_t*)(tk + H * H) + wave * (VT * 16 * VLD);  // this wave's V tile, transposed: [VT * 16 channels][VLD]
+  const int b = blockIdx.y;
+  const int q0 = a.cu_q[b], q1 = a.cu_q[b + 1];
+  const int t0 = q0 + ((int)gridDim.x - 1 - (int)blockIdx.x) * QR;
+  if (t0 >= q1) return;
+  const int tq = t0 + rq;
+  const bool qv = tq < q1;
+  const int64_t pq = qv ? a.positions[tq] : -1;
+  const int h0 = wave * HPW, gk = h0 / HG;
+  const uint16_t* q = (const uint16_t*)a.q;
+  const u32x4 zero4 = {0u, 0u, 0u, 0u};
+  u32x4 qf[HPW][DC];
+#pragma unroll
+  for (int hh = 0; hh < HPW; hh++)
+#pragma unroll
+    for (int c = 0; c < DC; c++) {
+      const int ch = c * 32 + oct * 8;
+      const bool ok = qv && ch < dim;
+      const u32x4 v = *(const u32x4*)(q + (size_t)(ok ? tq : q0) * a.ldq + (h0 + hh) * dim + (ok ? ch : 0));
+      qf[hh][c] = ok ? v : zero4;
+    }
+  long long lo = qv ? pq : 0x7fffffffffffffffll, hi = pq;  // (every wave holds the same 16 rows)
+  for (int o = 32; o > 0; o >>= 1) lo = min(lo, __shfl_xor(lo, o, 64)), hi = max(hi, __shfl_xor(hi, o, 64));
+  const int64_t pmin = lo, pmax = hi;
+  const int n_keys = (int)min((int64_t)a.context_lens[b], pmax + 1);
+  const int win = a.window;
+  const int keep_end = win > 0 ? (max(a.keep_first, 0) + KT - 1) / KT * KT : 0;
+  const int win_first = win > 0 ? (int)(max((int64_t)0, pmin - win + 1) / KT) * KT : 0;
+  auto next_tile = [&](int kt0) {
+    int n = kt0 + KT;
+    if (win > 0 && n >= keep_end && n < win_first) n = win_first;
+    return n;
+  };
+  for (int i = tid; i < H * H; i += 64 * NW) tk[i] = a.talk ? a.talk[i] : ((i / H == i % H) ? 1.f : 0.f);
+  const uint16_t* kc = (const uint16_t*)a.kc;
+  const uint16_t* vc = (const uint16_t*)a.vc;
+  const uint32_t* bt = a.block_tables + (size_t)b * a.max_blocks;
+  const int kdim = G * dim, vd_all = G * vdim;
+  f32x4 acc[HPW][VT];
+  float slope[HPW], hb[HPW];
+#pragma unroll
+  for (int hh = 0; hh < HPW; hh++) {
+    slope[hh] = a.slopes ? a.slopes[h0 + hh] : 0.f, hb[hh] = a.head_bias ? a.head_bias[h0 + hh] : 0.f;
+#pragma unroll
+    for (int t = 0; t < VT; t++) acc[hh][t] = vra_zero_acc();
+  }
+  // the wave's share of a tile: K fragments of its key/value head and that head's V tile ((pair of keys, 8 channels) items, 64 lanes)
+  constexpr int ITEMS = (KT / 2) * VT * 2, NV = ITEMS / 64;
+  static_assert(ITEMS % 64 == 0, "a wave's V items come in whole rounds");
+  u32x4 kfn[2][DC], vgn[NV][2];
+  auto page_slot = [&](int kt0) -> int64_t {
+    const int t = __builtin_amdgcn_readfirstlane(kt0);
+    return t < n_keys ? (int64_t)bt[t / a.BS] * a.BS + t % a.BS : 0;
+  };
+  // Requests carry no select: what lies outside the tile or the head is read from a valid address instead (slot 0, channel 0: finite
+  // numbers) and cannot reach a result — keys beyond the context get weight 0, channels beyond the key size meet zeros of the query
+  // fragment, channels beyond the value size are never stored.  So nothing has to wait for a request before the next one is issued.
+  auto request_tile = [&](int kt0, int64_t slot0) {
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+      const int key = kt0 + u * 16 + rq;
+      const uint16_t* kr = kc + (key < n_keys ? slot0 + (key - kt0) : 0) * kdim + gk * dim;
+#pragma unroll
+      for (int c = 0; c < DC; c++) {
+        const int ch = c * 32 + oct * 8;
+        kfn[u][c] = *(const u32x4*)(kr + (ch < dim ? ch : 0));
+      }
+    }
+#pragma unroll
+    for (int n = 0; n < NV; n++) {
+      const int i = lane + n * 64;
+      const int kp = i / (VT * 2), c8 = (i % (VT * 2)) * 8;
+#pragma unroll
+      for (int w2 = 0; w2 < 2; w2++) {
+        const int key = kt0 + kp * 2 + w2;
+        vgn[n][w2] = *(const u32x4*)(vc + (key < n_keys ? slot0 + (key - kt0) : 0) * vd_all + gk * vdim + (c8 < vdim ? c8 : 0));
+      }
+    }
+  };
+  int kt0 = (win > 0 && keep_end == 0 && win_first > 0) ? win_first : 0;
+  if (kt0 < n_keys) request_tile(kt0, page_slot(kt0));
+  while (kt0 < n_keys) {
+    const int ktn = next_tile(kt0);
+    const int64_t slot_next = page_slot(ktn);
+    // V tile -> this wave's LDS part, transposed, keys in the order the lanes hold their weights (the wave's earlier reads of it are done:
+    // LDS serves a wave's requests in order)
+    for (int n = 0; n < NV; n++) {
+      const int i = lane + n * 64;
+      if (i >= ITEMS) break;
+      const int kl = (i / (VT * 2)) * 2, c8 = (i % (VT * 2)) * 8;
+      const int pos = ((kl & 15) >> 2) * 8 + (kl >> 4) * 4 + (kl & 3);
+      uint32_t* row = (uint32_t*)vt;
+      for (int x = 0; x < 4; x++) {
+        const uint32_t lo0 = vgn[n][0][x] & 0xffffu, hi0 = vgn[n][0][x] >> 16, lo1 = vgn[n][1][x] & 0xffffu, hi1 = vgn[n][1][x] >> 16;
+        row[((c8 + 2 * x) * VLD + pos) >> 1] = lo0 | (lo1 << 16);
+        row[((c8 + 2 * x + 1) * VLD + pos) >> 1] = hi0 | (hi1 << 16);
+      }
+    }
+    // weights of the wave's own heads -> LDS
+#pragma unroll
+    for (int hh = 0; hh < HPW; hh++) {
+      f32x4 s[2];
+      s[0] = vra_zero_acc();
+      s[1] = vra_zero_acc();
+      for (int c = 0; c < DC; c++) {
+        BF16::mfma(s[0], __builtin_bit_cast(s16x8, kfn[0][c]), __builtin_bit_cast(s16x8, qf[hh][c]));
+        BF16::mfma(s[1], __builtin_bit_cast(s16x8, kfn[1][c]), __builtin_bit_cast(s16x8, qf[hh][c]));
+      }
+      VRA_MFMA_DRAIN();
+      f32x4 w4[2];
+      for (int u = 0; u < 2; u++)
+        for (int j = 0; j < 4; j++) {
+          const int key = kt0 + u * 16 + oct * 4 + j;
+          const int dist = (int)pq - key;  // (no short-circuit evaluation: the weights of a tile are straight-line code)
+          const bool seen = (dist >= 0) & (key < n_keys) & ((win <= 0) | (dist < win) | (key < a.keep_first));
+          const float x = s[u][j] * a.scale - slope[hh] * (float)dist + hb[hh];
+          w4[u][j] = seen ? __builtin_amdgcn_rcpf(1.f + __expf(-x)) : 0.f;  // (hardware exponential and reciprocal: no branches)
+        }
+      float* wr = wbuf + ((h0 + hh) * QR + rq) * WLD + oct * 8;
+      *(f32x4*)wr = w4[0];
+      *(f32x4*)(wr + 4) = w4[1];
+    }
+    if (ktn < n_keys) request_tile(ktn, slot_next);  // (on its way from memory during the meeting, the mix and the value products)
+    __syncthreads();
+    // mix: the wave's heads take their share of EVERY head's weight of the lane's (row, 8 keys)
+    float m[HPW][8];
+#pragma unroll
+    for (int hh = 0; hh < HPW; hh++)
+      for (int i = 0; i < 8; i++) m[hh][i] = 0.f;
+    for (int g = 0; g < H; g++) {
+      const float* wr = wbuf + (g * QR + rq) * WLD + oct * 8;
+      const f32x4 wa = *(const f32x4*)wr, wb = *(const f32x4*)(wr + 4);
+#pragma unroll
+      for (int hh = 0; hh < HPW; hh++) {
+        const float t = tk[(h0 + hh) * H + g];
+        for (int i = 0; i < 4; i++) m[hh][i] = fmaf(t, wa[i], m[hh][i]), m[hh][4 + i] = fmaf(t, wb[i], m[hh][4 + i]);
+      }
+    }
+    __syncthreads();
+    u32x4 vf[VT];
+#pragma unroll
+    for (int t = 0; t < VT; t++) vf[t] = *(const u32x4*)(vt + (t * 16 + rq) * VLD + oct * 8);
+#pragma unroll
+    for (int hh = 0; hh < HPW; hh++) {
+      u32x4 phi, plo;
+      for (int e = 0; e < 4; e++) {
+        const float a0 = m[hh][2 * e], a1 = m[hh][2 * e + 1];
+        const uint32_t hi2 = BF16::pack2(a0, a1);
+        phi[e] = hi2;
+        plo[e] = BF16::pack2(a0 - __uint_as_float(hi2 << 16), a1 - __uint_as_float(hi2 & 0xffff0000u));
+      }
+#pragma unroll
+      for (int t = 0; t < VT; t++) BF16::mfma(acc[hh][t], __builtin_bit_cast(s16x8, vf[t]), __builtin_bit_cast(s16x8, phi));
+#pragma unroll
+      for (int t = 0; t < VT; t++) BF16::mfma(acc[hh][t], __builtin_bit_cast(s16x8, vf[t]), __builtin_bit_cast(s16x8, plo));
+      VRA_MFMA_DRAIN();  // (per head: the compiler may park a head's accumulators elsewhere between tiles)
+    }
+    kt0 = ktn;
+  }
+  if (!qv) return;
+  uint16_t* out = (uint16_t*)a.out + (size_t)tq * H * vdim;
+#pragma unroll
+  for (int hh = 0; hh < HPW; hh++)
+#pragma unroll
+    for (int t = 0; t < VT; t++)
+      for (int j = 0; j < 4; j++) {
+        const int c = t * 16 + oct * 4 + j;
+        if (c >= vdim) continue;
+        float o = acc[hh][t][j];
+        if (a.gate) o *= sigmoidf_(a.gate[(size_t)tq * a.gate_ld + (h0 + hh) * vdim + c]);
+        out[(h0 + hh) * vdim + c] = BF16::from_f32(o);
+      }
 }
 
 // out[t, h, d] = sigmoid(gate[t, h, d]) * sum_g talk[h, g] U[t, g, kv(h), d]   (g ascending)
@@ -679,9 +867,42 @@ void vra_stack_sigmoid_attention(const StkSigAttnArgs& a, int dtype, int64_t str
       return;
     }
   }
-  if (!decode && dtype == VRA_BF16 && a.scratch && a.talk && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 128 && a.vdim <= 128 && a.ldq % 8 == 0 &&
-      ((uintptr_t)a.q % 16 == 0) && ((uintptr_t)a.kc % 16 == 0) && ((uintptr_t)a.vc % 16 == 0) && a.BS % 32 == 0 &&
-      (size_t)a.T * a.H * a.G * a.vdim * sizeof(float) <= a.scratch_bytes) {
+  const bool mfma_ok = !decode && dtype == VRA_BF16 && a.dim % 8 == 0 && a.vdim % 16 == 0 && a.dim <= 128 && a.vdim <= 128 && a.ldq % 8 == 0 &&
+                       ((uintptr_t)a.q % 16 == 0) && ((uintptr_t)a.kc % 16 == 0) && ((uintptr_t)a.vc % 16 == 0) && a.BS % 32 == 0;
+  // all heads in one workgroup: 4 waves of 1, 2 or 4 heads; a wave's heads share one key/value head
+  const int nw = 4, hpw = a.H / nw;
+  const bool per_head_ok = mfma_ok && a.scratch && a.talk && (size_t)a.T * a.H * a.G * a.vdim * sizeof(float) <= a.scratch_bytes;
+  // Its time follows the longest row block's key tiles, whatever the step's size (16 rows a workgroup: a 2048-token step is 128
+  // workgroups), the per-head kernel's follows the step's total work: measured at 16:4 heads of 128, 282 us against 395 at 2048 tokens,
+  // 154 against 101 at 512 — so short steps go to the per-head kernel when its scratch is there.
+  if (mfma_ok && (a.H == 4 || a.H == 8 || a.H == 16) && (a.H / a.G) % hpw == 0 && (a.T >= 1536 || !per_head_ok)) {
+    const int vt = (a.dim <= 64 && a.vdim <= 64) ? 4 : 8;
+    const size_t lds = ((size_t)a.H * 16 * 36 + (size_t)a.H * a.H) * sizeof(float) + (size_t)nw * vt * 16 * 40 * sizeof(uint16_t);
+    dim3 grid((a.max_q + 15) / 16, a.B);
+#define STK_SGH(DCV, VTV, HPWV, NWV)                                                                                                     \
+  do {                                                                                                                                    \
+    static bool attr = false;                                                                                                             \
+    if (!attr) {                                                                                                                          \
+      (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&stk_sig_prefill_heads_kernel<DCV, VTV, HPWV, NWV>),                        \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);                                                  \
+      attr = true;                                                                                                                        \
+    }                                                                                                                                     \
+    launch_checked("stack sigmoid attention (prefill, all heads)",                                                                        \
+                   [&] { stk_sig_prefill_heads_kernel<DCV, VTV, HPWV, NWV><<<grid, 64 * NWV, lds, st>>>(a); });                             \
+  } while (0)
+    if (vt == 4) {
+      if (a.H == 4) STK_SGH(2, 4, 1, 4);
+      else if (a.H == 8) STK_SGH(2, 4, 2, 4);
+      else STK_SGH(2, 4, 4, 4);
+    } else {
+      if (a.H == 4) STK_SGH(4, 8, 1, 4);
+      else if (a.H == 8) STK_SGH(4, 8, 2, 4);
+      else STK_SGH(4, 8, 4, 4);
+    }
+#undef STK_SGH
+    return;
+  }
+  if (per_head_ok) {
     const int gc = a.G >= 2 ? 2 : 1;  // value heads per workgroup: two keep the accumulators in registers, the scores are computed G / 2 times
     dim3 grid((a.max_q + 63) / 64, a.B, a.H * ((a.G + gc - 1) / gc));
 #define STK_SGM(DCV, VTV, GCV) launch_checked("stack sigmoid attention (prefill, mfma)", [&] { stk_sig_prefill_mfma_kernel<DCV, VTV, GCV><<<grid, 256, 0, st>>>(a, a.scratch); })

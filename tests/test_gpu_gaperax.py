@@ -48,19 +48,21 @@ def rnd(r, shape, sd=1.0):
 
 
 def freq_pair(rot):
-    """the rotary frequencies of `rot` as f32 hi + lo (the oracle's own table at position 1 gives the angles)"""
-    cos, sin = go.rotary_table(rot, [1])
-    mag = float(np.hypot(cos[0, 0], sin[0, 0])) if cos.size else 1.0
-    # angles below pi at position 1 only for the first pair of a table with base > 1: take the frequencies from the definition instead
+    """the rotary frequencies of `rot` as f32 hi + lo pairs and the factor on cos / sin, as the operators take them; formed here from the
+    definition and checked against the oracle's table at position 1"""
     dims, base = rot["dims"], rot["base"]
     i = np.arange(dims // 2, dtype=np.float64)
     f = base ** (-2.0 * i / dims)
+    mag = 1.0
     sc = rot.get("scaling")
     if sc:
-        td = lambda t: dims * math.log(sc["original"] / (2 * math.pi * t)) / (2 * math.log(base))
+        def td(t):
+            return dims * math.log(sc["original"] / (2 * math.pi * t)) / (2 * math.log(base))
         lo, hi = max(math.floor(td(sc["fast"])), 0), min(math.ceil(td(sc["slow"])), dims - 1)
         ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0, 1)
         f = f / sc["factor"] * ramp + f * (1 - ramp)
+        mag = 0.1 * math.log(sc["factor"]) + 1.0
+    cos, sin = go.rotary_table(rot, [1])
     assert np.allclose(np.cos(f) * mag, cos[0]) and np.allclose(np.sin(f) * mag, sin[0])
     fh = f.astype(np.float32)
     return fh, (f - fh.astype(np.float64)).astype(np.float32), mag

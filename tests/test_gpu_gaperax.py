@@ -644,3 +644,47 @@ def test_synthetic_weights_and_cache_plan():
     out = eng.generate([list(range(1, 40))], max_tokens=5, ignore_eos=True)[0]
     assert len(out) == 5
     eng.close()
+
+
+def test_trace_runner_on_a_model_folder(tmp_path):
+    """bin/trace_run as a user starts it: config.json + model.safetensors (bfloat16 tensors, scalar slopes of the norms as 0-d tensors) in a
+    folder, steps on standard input (a prompt in portions beside another request's single tokens, pages given back and taken again in a
+    pool of three), logits files out — against the oracle, in both dtypes"""
+    import json
+    import os
+    import struct
+    import subprocess
+    import sys
+    cfg = config_a()
+    tensors = go.random_tensors(cfg, 31)
+    model_dir = tmp_path / "model"
+    model_dir.mkdir()
+    (model_dir / "config.json").write_text(json.dumps(cfg))
+    header, blobs, off = {}, [], 0
+    for name, a in tensors.items():
+        b = checkpoint.f32_to_bf16_bits(np.asarray(a, np.float32)).tobytes()
+        header[name] = dict(dtype="BF16", shape=list(np.shape(a)), data_offsets=[off, off + len(b)])
+        off += len(b)
+        blobs.append(b)
+    h = json.dumps(header).encode()
+    (model_dir / "model.safetensors").write_bytes(struct.pack("<Q", len(h)) + h + b"".join(blobs))
+    p1, p2, p3 = tokens_of(cfg, 100, 1), tokens_of(cfg, 40, 2), tokens_of(cfg, 64, 3)
+    every = lambda n: list(range(n))
+    steps = [dict(entries=[dict(id="x", tokens=p1[:37], want=every(37)), dict(id="y", tokens=p2[:39], want=[])], end=[]),
+             dict(entries=[dict(id="x", tokens=p1[37:99], want=every(62)), dict(id="y", tokens=p2[39:], want=[0])], end=["y"]),
+             dict(entries=[dict(id="x", tokens=p1[99:], want=[0])], end=["x"]),
+             dict(entries=[dict(id="z", tokens=p3, want=every(64))], end=["z"])]
+    for i, s in enumerate(steps):
+        s["step"] = i
+    r1, r2, r3 = (go.forward(cfg, tensors, p) for p in (p1, p2, p3))
+    want = [r1[:37], np.concatenate([r1[37:99], r2[39:]]), r1[99:], r3]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dtype, dt in (("float32", F32), ("bfloat16", BF16)):
+        out = tmp_path / ("out_" + dtype)
+        r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", str(model_dir), "--dtype", dtype, "--out", str(out),
+                            "--max-tokens", "192"], input="\n".join(json.dumps(s) for s in steps).encode() + b"\n", capture_output=True, timeout=110)
+        assert r.returncode == 0, r.stderr.decode()[-1500:]
+        assert [ln for ln in r.stdout.decode().split("\n") if ln.startswith("done")] == ["done %d" % i for i in range(4)]
+        got = [np.fromfile(out / ("%d.f32" % i), "<f4").reshape(-1, cfg["vocab"]) for i in range(4)]
+        assert [g.shape[0] for g in got] == [w.shape[0] for w in want]
+        agree(np.concatenate(got), np.concatenate(want), dt, dtype)
